@@ -18,13 +18,15 @@ _runtime = None
 _runtime_err: Exception | None = None
 
 
-def _try_build() -> None:
+def _try_build(what: str = "all") -> None:
+    """Build one native module (or everything) in-tree; a process builds only
+    the module it is about to load."""
     if os.environ.get("DX_NO_AUTOBUILD"):
         return
     try:
         from . import build_native
 
-        build_native.build_all()
+        getattr(build_native, f"build_{what}")()
     except Exception as e:  # pragma: no cover - build env specific
         import sys
 
@@ -44,7 +46,7 @@ def kernels():
         try:
             _kernels = importlib.import_module("dynamo_exp_amd._C_kernels")
         except ImportError:
-            _try_build()
+            _try_build("kernels")
             try:
                 _kernels = importlib.import_module("dynamo_exp_amd._C_kernels")
             except ImportError as e:
@@ -54,6 +56,34 @@ def kernels():
                     "`python -m dynamo_exp_amd.build_native`"
                 ) from e
     return _kernels
+
+
+_mixers = None
+
+
+def mixers():
+    """Return the ``_C_mixers`` module (kernels of the layer-listed models),
+    building it in-tree on first use; raises when it cannot be had."""
+    global _mixers
+    if _mixers is not None:
+        return _mixers
+    with _lock:
+        if _mixers is not None:
+            return _mixers
+        import torch  # noqa: F401  -- torch's HIP runtime first
+
+        try:
+            _mixers = importlib.import_module("dynamo_exp_amd._C_mixers")
+        except ImportError:
+            _try_build("mixers")
+            try:
+                _mixers = importlib.import_module("dynamo_exp_amd._C_mixers")
+            except ImportError as e:
+                raise RuntimeError(
+                    "dynamo_exp_amd._C_mixers (gfx950 HIP kernels) is not built; run "
+                    "`python -m dynamo_exp_amd.build_native`"
+                ) from e
+    return _mixers
 
 
 def runtime():
@@ -67,7 +97,7 @@ def runtime():
         try:
             _runtime = importlib.import_module("dynamo_exp_amd._C_runtime")
         except ImportError:
-            _try_build()
+            _try_build("runtime")
             try:
                 _runtime = importlib.import_module("dynamo_exp_amd._C_runtime")
             except ImportError as e:

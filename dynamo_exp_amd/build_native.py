@@ -132,6 +132,37 @@ def build_kernels(verbose: bool = False, jobs: int = 8) -> Path:
     return out
 
 
+# every HIP source of this module is built without packed-fp32 instruction selection
+MIXER_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_mixers(verbose: bool = False, jobs: int = 8) -> Path:
+    """_C_mixers: the kernels of the layer-listed (hybrid) models
+    (csrc/mixers): multi-stream residual + norm, head prep + paged cache
+    write, row attention, gated activations.  A module of its own, so a
+    process that serves only such a model builds and loads nothing else."""
+    src_dir = CSRC / "mixers"
+    out = PKG / f"_C_mixers{EXT}"
+    objdir = BUILD / "mixers"
+    objdir.mkdir(parents=True, exist_ok=True)
+    srcs = sorted(src_dir.glob("*.hip")) + sorted(src_dir.glob("*.cpp"))
+    hdrs = _headers(src_dir) + [CSRC / "kernels" / "common.h"]
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    flags = _kernel_flags(src_dir)
+    objs, todo = [], []
+    for s in srcs:
+        o = objdir / (s.name + ".o")
+        objs.append(o)
+        if _stale(o, [s] + hdrs):
+            extra = ["-x", "hip", *MIXER_FLAGS] if s.suffix == ".hip" else []
+            todo.append([hipcc, *flags, *extra, "-c", str(s), "-o", str(o)])
+    with ThreadPoolExecutor(max(1, jobs)) as ex:
+        list(ex.map(lambda c: _run(c, verbose), todo))
+    if todo or _stale(out, objs):
+        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(out), *map(str, objs)], verbose)
+    return out
+
+
 def build_runtime(verbose: bool = False, jobs: int = 8) -> Path:
     src_dir = CSRC / "runtime"
     out = PKG / f"_C_runtime{EXT}"
@@ -191,7 +222,8 @@ def build_ctrld(verbose: bool = False) -> Path:
 def build_all(verbose: bool = False) -> list[Path]:
     jobs = int(os.environ.get("MAX_JOBS", "8"))
     jobs = max(1, min(jobs, 16))
-    return [build_runtime(verbose, jobs), build_capi(verbose), build_ctrld(verbose), build_kernels(verbose, jobs)]
+    return [build_runtime(verbose, jobs), build_capi(verbose), build_ctrld(verbose), build_kernels(verbose, jobs),
+            build_mixers(verbose, jobs)]
 
 
 if __name__ == "__main__":

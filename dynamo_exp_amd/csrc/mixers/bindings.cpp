@@ -1,0 +1,71 @@
+// pybind11 entry points of the layer-listed models' kernels (_C_mixers).
+// Raw device pointers (torch.Tensor.data_ptr()) and the HIP stream handle go
+// in; launches neither allocate nor synchronise, so they can be captured into
+// HIP graphs.  A launcher that rejects its arguments returns nonzero, raised
+// here.
+#include <hip/hip_runtime.h>
+#include <pybind11/pybind11.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+namespace py = pybind11;
+using u = uintptr_t;
+
+extern "C" {
+int dxm_stream_step(float*, const void*, int64_t, const float*, const float*, const float*, const float*, float, void*,
+                    int64_t, int, int, int, int, hipStream_t);
+int dxm_embed_streams(float*, const void*, const int64_t*, int, int, int, int64_t, int, hipStream_t);
+int dxm_glu_act(void*, const void*, int, int, int64_t, int64_t, int, int, hipStream_t);
+int dxm_headprep_cache(void*, int64_t, const int64_t*, const int64_t*, int, int, int, int, int, const float*,
+                       const float*, float, float, double, void*, void*, int, int, int, int, hipStream_t);
+int dxm_diff_combine(void*, const float*, int64_t, int, float, float, float, int, hipStream_t);
+int dxm_row_attention(void*, float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*,
+                      const int*, int, int, int, int, int, int, int, int, int, int, float, int, int, int, int, int,
+                      hipStream_t);
+}
+
+static void check(int rc, const char* what) {
+  if (rc != 0) throw std::runtime_error(std::string(what) + " rejected its arguments (code " + std::to_string(rc) + ")");
+}
+
+#define P(x) reinterpret_cast<void*>(x)
+#define F(x) reinterpret_cast<float*>(x)
+#define S(x) reinterpret_cast<hipStream_t>(x)
+
+PYBIND11_MODULE(_C_mixers, m) {
+  m.doc() = "dynamo_exp_amd gfx950 kernels of layer-listed models";
+  m.attr("arch") = "gfx950";
+  m.def("stream_step", [](u X, u y, int64_t ys, u mix, u gain, u rin, u nw, float eps, u out, int64_t os, int rows,
+                          int S_, int W, int f32, u st) {
+    check(dxm_stream_step(F(X), P(y), ys, F(mix), F(gain), F(rin), F(nw), eps, P(out), os, rows, S_, W, f32, S(st)),
+          "stream_step");
+  });
+  m.def("embed_streams", [](u X, u table, u ids, int rows, int S_, int W, int64_t vocab, int f32, u st) {
+    check(dxm_embed_streams(F(X), P(table), reinterpret_cast<const int64_t*>(ids), rows, S_, W, vocab, f32, S(st)),
+          "embed_streams");
+  });
+  m.def("glu_act", [](u out, u gu, int rows, int Fw, int64_t is, int64_t os, int act, int f32, u st) {
+    check(dxm_glu_act(P(out), P(gu), rows, Fw, is, os, act, f32, S(st)), "glu_act");
+  });
+  m.def("headprep_cache", [](u x, int64_t xs, u pos, u slots, int rows, int n_q, int n_k, int d, int k_off, u qw, u kw,
+                             float eps, float coef, double every, u kc, u vc, int v_mode, int v_off, int v_w, int f32,
+                             u st) {
+    check(dxm_headprep_cache(P(x), xs, reinterpret_cast<const int64_t*>(pos), reinterpret_cast<const int64_t*>(slots),
+                             rows, n_q, n_k, d, k_off, F(qw), F(kw), eps, coef, every, P(kc), P(vc), v_mode, v_off,
+                             v_w, f32, S(st)),
+          "headprep_cache");
+  });
+  m.def("diff_combine", [](u out, u a, int64_t n_vec, int dv, float lam, float post, float eps, int f32, u st) {
+    check(dxm_diff_combine(P(out), F(a), n_vec, dv, lam, post, eps, f32, S(st)), "diff_combine");
+  });
+  m.def("row_attention", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
+                            int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
+                            int size, int parts, int f32, int out_f32, u st) {
+    check(dxm_row_attention(P(out), F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
+                            reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
+                            maps, group, d, dv, Wk, Wv, scale, mask, size, parts, f32, out_f32, S(st)),
+          "row_attention");
+  });
+}

@@ -1,0 +1,280 @@
+// Row-wise kernels of layer-listed (hybrid) models on gfx950: the multi-stream
+// residual ("hyper-connections") update fused with the next sublayer's
+// read-in and RMS norm, the embedding gather into fp32 streams, gated
+// feed-forward activations, per-head q/k normalisation fused with the paged
+// cache write, and the two-map (differential) attention combine.
+//
+// Every kernel is a template over the activation element (bf16 bits or
+// float); reductions, norms, the residual streams and every scale are fp32
+// whatever the element is.  Sizes are run-time arguments: nothing here is
+// specialised for one model's widths.
+#include "../kernels/common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxStreams = 8;
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+
+// One residual step of a model with S parallel residual streams X [rows, S, W]
+// (fp32, updated in place).  With y (the previous sublayer's output):
+//     X_t <- sum_s mix[s, t] X_s + gain[t] * y          for every stream t
+// then, with read-in weights rin [S]:  u = sum_s rin[s] X_s  and
+//     out = u / sqrt(mean(u^2) + eps) * nw              (nw fp32 [W]; nw == null: out = u)
+// S = 1, mix = [1], gain = [1], rin = [1] is the ordinary pre-norm residual.
+template <typename T>
+__global__ void __launch_bounds__(kThreads) stream_step_kernel(float* __restrict__ X, const T* __restrict__ y,
+                                                               int64_t y_stride, const float* __restrict__ mix,
+                                                               const float* __restrict__ gain,
+                                                               const float* __restrict__ rin,
+                                                               const float* __restrict__ nw, float eps,
+                                                               T* __restrict__ out, int64_t out_stride, int S, int W) {
+  __shared__ float red[16];
+  __shared__ float sm[kMaxStreams * kMaxStreams + 2 * kMaxStreams];
+  const int64_t row = blockIdx.x;
+  float* x = X + row * (int64_t)S * W;
+  float* s_mix = sm;
+  float* s_gain = sm + kMaxStreams * kMaxStreams;
+  float* s_in = s_gain + kMaxStreams;
+  if (threadIdx.x < S * S && y) s_mix[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    s_gain[threadIdx.x] = y ? gain[threadIdx.x] : 0.f;
+    s_in[threadIdx.x] = rin ? rin[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += kThreads) {
+    float v[kMaxStreams];
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s) v[s] = s < S ? x[(int64_t)s * W + c] : 0.f;
+    if (y) {
+      const float yv = ldf<T>(y, row * y_stride + c);
+      float n[kMaxStreams];
+#pragma unroll
+      for (int t = 0; t < kMaxStreams; ++t) {
+        float a = 0.f;
+        if (t < S) {
+#pragma unroll
+          for (int s = 0; s < kMaxStreams; ++s)
+            if (s < S) a += s_mix[s * S + t] * v[s];
+          a += s_gain[t] * yv;
+          x[(int64_t)t * W + c] = a;
+        }
+        n[t] = a;
+      }
+#pragma unroll
+      for (int t = 0; t < kMaxStreams; ++t) v[t] = n[t];
+    }
+    if (rin) {
+      float uu = 0.f;
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s)
+        if (s < S) uu += s_in[s] * v[s];
+      ss += uu * uu;
+    }
+  }
+  if (!rin) return;
+  const float tot = block_reduce_sum(ss, red);
+  const float r = nw ? rsqrtf(tot / (float)W + eps) : 1.f;
+  // second pass: this thread re-reads the stream values it wrote itself
+  for (int c = threadIdx.x; c < W; c += kThreads) {
+    float uu = 0.f;
+    for (int s = 0; s < S; ++s) uu += s_in[s] * x[(int64_t)s * W + c];
+    stf<T>(out, row * out_stride + c, nw ? uu * r * nw[c] : uu);
+  }
+}
+
+// X[t, s, :] = table[ids[t], :] for every stream s (fp32 streams)
+template <typename T>
+__global__ void __launch_bounds__(kThreads) embed_streams_kernel(float* __restrict__ X, const T* __restrict__ table,
+                                                                 const int64_t* __restrict__ ids, int S, int W,
+                                                                 int64_t vocab) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = ids[t];
+  const bool ok = id >= 0 && id < vocab;
+  for (int c = threadIdx.x; c < W; c += kThreads) {
+    const float v = ok ? ldf<T>(table, id * (int64_t)W + c) : 0.f;
+    for (int s = 0; s < S; ++s) X[(t * S + s) * (int64_t)W + c] = v;
+  }
+}
+
+__device__ __forceinline__ float act_fn(float z, int act) {
+  if (act == 0) return fmaxf(z, 0.f);           // relu
+  if (act == 1) return z / (1.f + __expf(-z));  // silu
+  const float c = 0.7978845608028654f;          // gelu, tanh form
+  return 0.5f * z * (1.f + tanhf(c * (z + 0.044715f * z * z * z)));
+}
+
+// gu [rows, 2F] = [gate | up]  ->  out [rows, F] = act(gate) * up
+template <typename T>
+__global__ void __launch_bounds__(kThreads) glu_act_kernel(T* __restrict__ out, const T* __restrict__ gu, int F,
+                                                           int64_t in_stride, int64_t out_stride, int act) {
+  const int64_t r = blockIdx.y;
+  for (int c = blockIdx.x * kThreads + threadIdx.x; c < F; c += gridDim.x * kThreads) {
+    const float g = ldf<T>(gu, r * in_stride + c), u = ldf<T>(gu, r * in_stride + F + c);
+    stf<T>(out, r * out_stride + c, act_fn(g, act) * u);
+  }
+}
+
+// Per token row of a fused projection output x = [q | k | v]:
+//   q: n_q vectors of d; with qw: unit RMS times qw [d]; with temp_coef != 0 a
+//      position-dependent gain 1 + coef * ln(floor((p + 1) / every) + 1); in place
+//   k: n_k vectors of d at column k_off; with kw: unit RMS times kw; written to
+//      the K cache row of the token's slot (kc [slots, n_k * d])
+//   v: v_mode 0: no V cache (V is the K cache); 1: the k section as projected
+//      (before its norm) is the value; 2: v_w columns at v_off are the value
+// slot < 0: nothing is cached for the row.  One wave per vector.
+template <typename T>
+__global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
+    T* __restrict__ x, int64_t x_stride, const int64_t* __restrict__ pos, const int64_t* __restrict__ slots,
+    int n_q, int n_k, int d, int k_off, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    float temp_coef, double temp_every, T* __restrict__ kc, T* __restrict__ vc, int v_mode, int v_off, int v_w) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = kThreads / 64;
+  T* row = x + t * x_stride;
+  const int64_t slot = slots[t];
+  const int k_w = n_k * d;
+  float gain = 1.f;
+  if (temp_coef != 0.f) {
+    const double k = floor((double)(pos[t] + 1) / temp_every);
+    gain = 1.f + temp_coef * logf((float)k + 1.f);
+  }
+  const bool q_work = qw != nullptr || temp_coef != 0.f;
+  for (int v = wid; v < n_q + n_k; v += nw) {
+    const bool is_q = v < n_q;
+    if (is_q && !q_work) continue;
+    if (!is_q && slot < 0) continue;
+    T* src = is_q ? row + (int64_t)v * d : row + k_off + (int64_t)(v - n_q) * d;
+    const float* w = is_q ? qw : kw;
+    float r = 1.f;
+    if (w) {
+      float ss = 0.f;
+      for (int e = lane; e < d; e += 64) {
+        const float a = ldf<T>(src, e);
+        ss += a * a;
+      }
+      r = rsqrtf(wave_reduce_sum(ss) / (float)d + eps);
+    }
+    if (is_q) {
+      for (int e = lane; e < d; e += 64) stf<T>(src, e, ldf<T>(src, e) * (w ? r * w[e] : 1.f) * gain);
+    } else {
+      T* kd = kc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d;
+      T* vd = v_mode == 1 ? vc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d : nullptr;
+      for (int e = lane; e < d; e += 64) {
+        const float a = ldf<T>(src, e);
+        if (vd) vd[e] = src[e];
+        stf<T>(kd, e, w ? a * r * w[e] : a);
+      }
+    }
+  }
+  if (v_mode == 2 && slot >= 0) {
+    const T* vs = row + v_off;
+    T* vd = vc + slot * (int64_t)v_w;
+    for (int e = threadIdx.x; e < v_w; e += kThreads) vd[e] = vs[e];
+  }
+}
+
+// Two-map attention combine: a [rows, H, 2, dv] fp32 (map outputs over the
+// same values)  ->  out [rows, H, dv] = unit_rms(a1 - lam * a2) * post.
+// One wave per (row, head).
+template <typename T>
+__global__ void __launch_bounds__(kThreads) diff_combine_kernel(T* __restrict__ out, const float* __restrict__ a,
+                                                                int64_t n_vec, int dv, float lam, float post,
+                                                                float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t v = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+  if (v >= n_vec) return;
+  const float* a1 = a + v * 2 * (int64_t)dv;
+  const float* a2 = a1 + dv;
+  float ss = 0.f;
+  for (int e = lane; e < dv; e += 64) {
+    const float o = a1[e] - lam * a2[e];
+    ss += o * o;
+  }
+  const float r = rsqrtf(wave_reduce_sum(ss) / (float)dv + eps) * post;
+  for (int e = lane; e < dv; e += 64) stf<T>(out, v * dv + e, (a1[e] - lam * a2[e]) * r);
+}
+
+}  // namespace
+
+#define DISPATCH_T(f32, ...)          \
+  if (f32) {                          \
+    using T = float;                  \
+    __VA_ARGS__;                      \
+  } else {                            \
+    using T = bf16_t;                 \
+    __VA_ARGS__;                      \
+  }
+
+extern "C" {
+
+int dxm_stream_step(float* X, const void* y, int64_t y_stride, const float* mix, const float* gain, const float* rin,
+                    const float* nw, float eps, void* out, int64_t out_stride, int rows, int S, int W, int f32,
+                    hipStream_t st) {
+  if (S < 1 || S > kMaxStreams || W < 1) return 1;
+  if (rows <= 0) return 0;
+  if (y && (!mix || !gain)) return 2;
+  if (rin && !out) return 3;
+  DISPATCH_T(f32, hipLaunchKernelGGL(stream_step_kernel<T>, dim3(rows), dim3(kThreads), 0, st, X, (const T*)y,
+                                     y_stride, mix, gain, rin, nw, eps, (T*)out, out_stride, S, W));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_embed_streams(float* X, const void* table, const int64_t* ids, int rows, int S, int W, int64_t vocab, int f32,
+                      hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH_T(f32, hipLaunchKernelGGL(embed_streams_kernel<T>, dim3(rows), dim3(kThreads), 0, st, X, (const T*)table,
+                                     ids, S, W, vocab));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_glu_act(void* out, const void* gu, int rows, int F, int64_t in_stride, int64_t out_stride, int act, int f32,
+                hipStream_t st) {
+  if (rows <= 0 || F <= 0) return 0;
+  if (act < 0 || act > 2) return 1;
+  const int gx = (F + kThreads - 1) / kThreads;
+  for (int r0 = 0; r0 < rows; r0 += 65535) {
+    const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
+    DISPATCH_T(f32, hipLaunchKernelGGL(glu_act_kernel<T>, dim3(gx, nr), dim3(kThreads), 0, st,
+                                       (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
+                                       out_stride, act));
+  }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int64_t* slots, int rows, int n_q, int n_k,
+                       int d, int k_off, const float* qw, const float* kw, float eps, float temp_coef,
+                       double temp_every, void* kc, void* vc, int v_mode, int v_off, int v_w, int f32,
+                       hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (n_q < 0 || n_k < 0 || d < 1 || v_mode < 0 || v_mode > 2) return 1;
+  if (n_k > 0 && !kc) return 2;
+  if (v_mode != 0 && !vc) return 3;
+  if (temp_coef != 0.f && !(temp_every > 0)) return 4;
+  DISPATCH_T(f32, hipLaunchKernelGGL(headprep_cache_kernel<T>, dim3(rows), dim3(kThreads), 0, st, (T*)x, x_stride, pos,
+                                     slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every, (T*)kc, (T*)vc,
+                                     v_mode, v_off, v_w));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_diff_combine(void* out, const float* a, int64_t n_vec, int dv, float lam, float post, float eps, int f32,
+                     hipStream_t st) {
+  if (n_vec <= 0) return 0;
+  const int64_t blocks = (n_vec + kThreads / 64 - 1) / (kThreads / 64);
+  DISPATCH_T(f32, hipLaunchKernelGGL(diff_combine_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, st, (T*)out, a,
+                                     n_vec, dv, lam, post, eps));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // extern "C"

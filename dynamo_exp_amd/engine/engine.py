@@ -28,6 +28,7 @@ import torch
 
 from ..models.config import ModelConfig, get_config
 from ..models.llama import LlamaForCausalLM, TPGroup
+from ..models.registry import build_model
 from ..runtime.chan import Chan
 from ..utils import streams, tracing
 from ..utils.faults import FAULTS
@@ -73,6 +74,9 @@ class EngineConfig:
     # scales kv_scales; halves the KV bytes decode attention streams)
     kv_cache_dtype: str = "auto"
     kv_scales: tuple = (1.0, 1.0)
+    # activation / weight dtype: "bfloat16", or "float32" for the models that
+    # have true 32-bit kernels (models/registry.py)
+    dtype: str = "bfloat16"
     # the KV cache is written by peer processes (decode engine behind the
     # one-sided "ipc" KV transport): allocate it shareable (disagg/kv_share.py)
     kv_shared: bool = os.environ.get("DX_KV_SHARED", "0") == "1"
@@ -106,7 +110,7 @@ class LLMEngine:
             cfg.max_model_len = self.model_cfg.max_position_embeddings
         dev = torch.device(cfg.device)
         if model is None:
-            model = LlamaForCausalLM(self.model_cfg, device=dev, tp=tp)
+            model = build_model(self.model_cfg, device=dev, tp=tp, dtype=cfg.dtype)
             if cfg.random_init or not os.path.isdir(cfg.model):
                 model.random_init(cfg.seed)
             else:
@@ -313,6 +317,35 @@ class LLMEngine:
     def has_pending_work(self) -> bool:
         """Whether step() would do anything now."""
         return self.scheduler.has_work() or self._inflight is not None
+
+    # ---------------------------------------------------------------- forced steps
+    def forced_step(self, entries: list[tuple[str, list[int], list[int]]], end: list[str] | None = None) -> dict:
+        """Feed given tokens instead of sampling (trace replay, scoring): one
+        engine step over `entries` = (request id, next tokens, offsets among
+        them whose logits are wanted), all in one batch through the scheduler's
+        page management and the runner's forward.  Requests in `end` are
+        finished afterwards.  Returns {request id: fp32 logits [n_wanted,
+        vocab]} for entries that wanted any."""
+        if self._cuda:
+            streams.enter_compute(self.model.device)
+        if self._inflight is not None:
+            raise RuntimeError("forced_step with a sampled batch in flight")
+
+        def new_request(rid: str) -> Request:
+            req = Request(rid, [], SamplingParams(max_tokens=1, ignore_eos=True))
+            self.requests[rid] = req
+            return req
+
+        batch = self.scheduler.schedule_forced(entries, new_request)
+        self.last_batch = batch
+        logits = self.runner.score(batch)
+        self.scheduler.update_forced(batch, list(end or []))
+        for rid in end or []:
+            self.requests.pop(rid, None)
+        self.stats["steps"] += 1
+        self.stats[f"{batch.kind}_steps"] += 1
+        self.stats["prompt_tokens"] += batch.num_tokens
+        return {r.request_id: lg for r, lg in zip(batch.requests, logits) if lg.shape[0]}
 
     # ---------------------------------------------------------------- step
     def step(self) -> list[Request]:

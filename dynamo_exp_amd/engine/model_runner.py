@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..models.llama import AttnMeta, LlamaForCausalLM
+from ..models.llama import AttnMeta, LlamaForCausalLM  # noqa: F401 -- any registered model class fits
 from .request import Request
 
 # device-time accounting with CUDA events around each launch (DX_GPU_TIMING=0: off)
@@ -76,11 +76,23 @@ class ModelRunner:
         # reserved out of the KV budget (it used to grow unbounded)
         self.kv_fp8 = cfg.kv_dtype == torch.float8_e4m3fn
         self.fp8_scratch_cap = max(2 * self.max_blocks_per_seq, 256) if self.kv_fp8 else 0
+        # models that lay out their own caches (per layer run, K and V rows of
+        # their own widths: models/bekulix.py) and take one attention launch
+        # over all rows of a step
+        self.unified = bool(getattr(model, "unified_rows", False))
         self.num_blocks = cfg.num_gpu_blocks or self._auto_blocks()
         L = mc.num_hidden_layers
-        shape = (L, 2, self.num_blocks, model.n_kv, cfg.block_size, model.head_dim)
         self.kv_share = None
-        if cfg.kv_shared and self.is_gpu:
+        if self.unified:
+            if self.kv_fp8 or cfg.kv_shared:
+                raise ValueError(f"{type(model).__name__}: fp8 / peer-shared KV caches are not available")
+            self.kv_cache = None
+            self.kv_caches = model.alloc_kv_caches(self.num_blocks, cfg.block_size, model.dtype)
+        else:
+            shape = (L, 2, self.num_blocks, model.n_kv, cfg.block_size, model.head_dim)
+        if self.unified:
+            pass
+        elif cfg.kv_shared and self.is_gpu:
             from ..disagg.kv_share import SharedKVBuffer
 
             nbytes = math.prod(shape) * torch.empty((), dtype=cfg.kv_dtype).element_size()
@@ -89,7 +101,8 @@ class ModelRunner:
             self.kv_cache.zero_()
         else:
             self.kv_cache = torch.zeros(shape, dtype=cfg.kv_dtype, device=self.device)
-        self.kv_caches = [(self.kv_cache[i, 0], self.kv_cache[i, 1]) for i in range(L)]
+        if not self.unified:
+            self.kv_caches = [(self.kv_cache[i, 0], self.kv_cache[i, 1]) for i in range(L)]
         self.graphs: dict[int, tuple] = {}
         self.graphs_sharded: dict[int, object] = {}  # TP > 1: vocab-sharded sampler variant
         self._res_tok = self._res_lp = None  # multi-step decode result buffers
@@ -110,8 +123,11 @@ class ModelRunner:
     # ------------------------------------------------------------------ memory
     def _auto_blocks(self) -> int:
         mc = self.model.cfg
-        per_block = (mc.num_hidden_layers * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim *
-                     torch.empty((), dtype=self.cfg.kv_dtype).element_size())
+        if self.unified:
+            per_block = self.model.kv_bytes_per_block(self.cfg.block_size, self.model.dtype)
+        else:
+            per_block = (mc.num_hidden_layers * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim *
+                         torch.empty((), dtype=self.cfg.kv_dtype).element_size())
         if not self.is_gpu:
             return max(64, (256 << 20) // per_block)
         free, total = torch.cuda.mem_get_info(self.device)
@@ -119,7 +135,8 @@ class ModelRunner:
         # activations / graphs / logits headroom
         budget -= 6 << 30
         # fp8 prefill dequant scratch (bf16 K + V, one layer at a time)
-        budget -= self.fp8_scratch_cap * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim * 2
+        if self.fp8_scratch_cap:
+            budget -= self.fp8_scratch_cap * 2 * self.model.n_kv * self.cfg.block_size * self.model.head_dim * 2
         n = int(budget // per_block)
         if n <= 0:
             raise RuntimeError("not enough GPU memory for the KV cache")
@@ -127,6 +144,8 @@ class ModelRunner:
 
     @property
     def kv_bytes(self) -> int:
+        if self.unified:
+            return sum(t.numel() * t.element_size() for k, v in self.kv_caches for t in ((k,) if v is k else (k, v)))
         return self.kv_cache.numel() * self.kv_cache.element_size()
 
     def block_bytes_per_layer(self) -> int:
@@ -184,15 +203,20 @@ class ModelRunner:
             pos.append(d_pos)
             slots.append(d_slots)
             rows.extend(range(Tp, Tp + B))
-            dmeta = AttnMeta(is_prefill=False, positions=None, slot_mapping=None,
-                             block_tables=self._to_dev(self._block_table(decode), torch.int32),
-                             ctx_lens=self._to_dev(d_ctx, torch.int32), n_parts=self._n_parts(B))
-            if self.is_gpu:
+            if self.unified:
+                ctx = ctx + [int(c) for c in d_ctx]
+            else:
+                dmeta = AttnMeta(is_prefill=False, positions=None, slot_mapping=None,
+                                 block_tables=self._to_dev(self._block_table(decode), torch.int32),
+                                 ctx_lens=self._to_dev(d_ctx, torch.int32), n_parts=self._n_parts(B))
+            if self.is_gpu and not self.unified:
                 dmeta.workspace = ops.decode_workspace(B, self.model.n_q, self.model.head_dim, dmeta.n_parts,
                                                        self.device)
         pos = np.concatenate(pos)
         slots = np.concatenate(slots)
         mc = self.model
+        if self.unified:
+            return self._unified_meta(ids, pos, slots, reqs, num_new, decode or [], cu, ctx, rows)
         work = ops.prefill_work_list(num_new, ctx, mc.n_q, mc.n_kv) if reqs else []
         meta = AttnMeta(
             is_prefill=True,
@@ -211,6 +235,29 @@ class ModelRunner:
         if mm_rows:
             meta.mm_rows = self._to_dev(np.asarray(mm_rows, dtype=np.int64), torch.int64)
             meta.mm_embeds = torch.cat(mm_parts) if len(mm_parts) > 1 else mm_parts[0]
+        return self._to_dev(np.asarray(ids, dtype=np.int64), torch.int64), meta
+
+    def _unified_meta(self, ids, pos, slots, reqs, num_new, decode, cu, ctx, rows):
+        """Step metadata of a `unified_rows` model: every row (prompt-chunk
+        tokens, then one row per decode request) names its sequence, a row of
+        the stacked block table."""
+        allr = list(reqs) + list(decode)
+        seq = np.concatenate([np.repeat(np.arange(len(reqs), dtype=np.int32), num_new),
+                              np.arange(len(reqs), len(allr), dtype=np.int32)])
+        meta = AttnMeta(
+            is_prefill=True,
+            positions=self._to_dev(pos, torch.int64),
+            slot_mapping=self._to_dev(slots, torch.int64),
+            block_tables=None,
+            ctx_lens=None,
+            cu_seqlens_q=self._to_dev(np.asarray(cu, dtype=np.int32), torch.int32),
+            logits_idx=self._to_dev(np.asarray(rows, dtype=np.int64), torch.int64),
+            num_prefill_tokens=cu[-1],
+            row_seq=self._to_dev(seq, torch.int32),
+            row_tables=self._to_dev(self._block_table(allr), torch.int32),
+            block_size=self.block_size,
+            max_ctx=max(ctx) if ctx else 0,
+        )
         return self._to_dev(np.asarray(ids, dtype=np.int64), torch.int64), meta
 
     def _plan_fp8_scratch(self, meta, reqs, num_new, ctx, cu) -> None:
@@ -327,6 +374,33 @@ class ModelRunner:
             out.event.record()
         return out
 
+    @torch.inference_mode()
+    def score(self, batch) -> list[torch.Tensor]:
+        """Run a forced batch (scheduler.schedule_forced: the tokens are given,
+        nothing is sampled) and return, per request in batch order, the fp32
+        logits [len(want_i), vocab] at the offsets batch.want[i] of the tokens
+        the request computes in this step."""
+        npre = batch.n_prefill
+        reqs, decode = batch.requests[:npre], batch.requests[npre:]
+        ids, meta = self.prepare_prefill(reqs, batch.num_new, [False] * npre, decode)
+        rows, counts, t0 = [], [], 0
+        for i, r in enumerate(batch.requests):
+            n = batch.num_new[i] if i < npre else 1
+            w = batch.want[i]
+            if any(not 0 <= o < n for o in w):
+                raise ValueError(f"{r.request_id}: wanted offsets {w} outside the {n} tokens of this step")
+            rows.extend(t0 + o for o in w)
+            counts.append(len(w))
+            t0 += n
+        meta.logits_idx = self._to_dev(np.asarray(rows, dtype=np.int64), torch.int64)
+        hidden = self.model.forward(ids, meta, self.kv_caches)
+        self.timing["prefill_tokens"] += sum(batch.num_new)
+        self.timing["prefill_steps"] += 1
+        if not rows:
+            return [hidden.new_empty((0, self.vocab), dtype=torch.float32) for _ in counts]
+        logits = self.model.compute_logits(hidden, fp32=True)
+        return list(logits.split(counts, 0))
+
     def fetch(self, h: Launched) -> tuple[list[int], list[float]]:
         """Host values of a launched batch's tokens (waits for them)."""
         t1 = time.perf_counter()
@@ -419,9 +493,11 @@ class ModelRunner:
             slot_mapping=self._to_dev(slots, torch.int64),
             block_tables=self._to_dev(self._block_table(reqs), torch.int32),
             ctx_lens=self._to_dev(ctx, torch.int32),
-            n_parts=self._n_parts(B),
+            n_parts=1 if self.unified else self._n_parts(B),
+            block_size=self.block_size,
+            max_ctx=int(ctx.max()) if B else 0,
         )
-        if self.is_gpu:
+        if self.is_gpu and not self.unified:
             meta.workspace = ops.decode_workspace(B, self.model.n_q, self.model.head_dim, meta.n_parts, self.device)
         ids_t = self._to_dev(ids, torch.int64)
         if patch:
@@ -487,8 +563,8 @@ class ModelRunner:
         self._out_tok = torch.zeros(maxB, dtype=torch.int64, device=dev)
         self._out_lp = torch.zeros(maxB, dtype=torch.float32, device=dev)
         # one flat decode-attention workspace, viewed per bucket as [B, Hq, P(B), ...]
-        ws = max(B * self._n_parts(B) for B in self.cfg.graph_sizes)
-        self._workspace = (torch.empty(ws * self.model.n_q * self.model.head_dim, dtype=torch.float32, device=dev),
+        ws = 0 if self.unified else max(B * self._n_parts(B) for B in self.cfg.graph_sizes)
+        self._workspace = None if self.unified else (torch.empty(ws * self.model.n_q * self.model.head_dim, dtype=torch.float32, device=dev),
                            torch.empty(ws * self.model.n_q * 2, dtype=torch.float32, device=dev))
         self._static = True
 
@@ -503,8 +579,10 @@ class ModelRunner:
             slot_mapping=dv["slots"][:B],
             block_tables=dv["bt"][:B],
             ctx_lens=dv["ctx"][:B],
-            n_parts=self._n_parts(B),
-            workspace=self._graph_workspace(B),
+            n_parts=1 if self.unified else self._n_parts(B),
+            workspace=None if self.unified else self._graph_workspace(B),
+            block_size=self.block_size,
+            max_ctx=self.cfg.max_model_len,
         )
         hidden = self.model.forward(dv["ids"][:B], meta, self.kv_caches)
         if not full:

@@ -81,6 +81,9 @@ class Batch:
     num_new: list[int] = field(default_factory=list)
     sample: list[bool] = field(default_factory=list)
     epochs: list[int] = field(default_factory=list)  # async: Request.epoch of `sampled` at launch
+    # forced (teacher-fed) batches: per request, the offsets among the tokens it
+    # computes in this step whose logits are wanted; nothing is sampled
+    want: list[list[int]] | None = None
 
     @property
     def n_prefill(self) -> int:
@@ -107,6 +110,7 @@ class Scheduler:
         self.remote: dict[str, Request] = {}  # REMOTE_PREFILLING on the decode side
         self.transferring: dict[str, Request] = {}  # prefill side: KV handed to a decode worker
         self.reading: dict[str, Request] = {}  # prefill side: pulling a cached prefix (READ path)
+        self.forced: dict[str, Request] = {}  # live requests of forced steps (schedule_forced)
         # decode side, one-sided (IPC) KV transport: remote prefills whose KV a
         # prefill worker may be writing straight into their blocks, and the ones
         # aborted meanwhile, whose blocks are held until that write is done
@@ -517,6 +521,56 @@ class Scheduler:
             self._append_token(r, tok, lp)
             out.append(r)
         return out
+
+    # ------------------------------------------------------------------ forced (teacher-fed) steps
+    def schedule_forced(self, entries: list[tuple[str, list[int], list[int]]], new_request) -> Batch:
+        """One step whose tokens are given from outside (trace replay,
+        scoring): `entries` = (request id, the request's next tokens, wanted
+        offsets).  An unknown id is admitted (`new_request(id)` makes the
+        Request), a known one continues where its last step ended.  Entries of
+        several tokens run as prompt chunks, a single token after the first
+        step as a decode row; all of them form one batch.  Pages come from the
+        KV manager as for any request; an exhausted pool raises (a forced step
+        never preempts)."""
+        pre, dec = [], []
+        for rid, toks, want in entries:
+            if not toks:
+                raise ValueError(f"{rid}: a step entry needs at least one token")
+            r = self.forced.get(rid)
+            if r is None:
+                if len(self.forced) + len(self.running) + len(self.prefilling) >= self.cfg.max_num_seqs:
+                    raise RuntimeError(f"{rid}: more than max_num_seqs={self.cfg.max_num_seqs} live requests")
+                r = self.forced[rid] = new_request(rid)
+                r.status = Status.RUNNING
+                r.admit_time = time.perf_counter()
+            if r.num_tokens + len(toks) > self.cfg.max_model_len:
+                raise ValueError(f"{rid}: {r.num_tokens + len(toks)} tokens exceed max_model_len")
+            if not self.kv.ensure_slots(r, r.num_tokens + len(toks)):
+                raise RuntimeError(f"{rid}: KV pool exhausted ({self.kv.num_free()} blocks free)")
+            if len(toks) == 1 and r.num_tokens > 0:
+                r.output.append(int(toks[0]))
+                dec.append((r, list(want)))
+            else:
+                if r.output:  # earlier single tokens become part of the prompt
+                    r.prompt = r.prompt + r.output
+                    r.output = []
+                r.prompt = r.prompt + [int(t) for t in toks]
+                pre.append((r, len(toks), list(want)))
+        kind = "mixed" if pre and dec else ("prefill" if pre else "decode")
+        return Batch(kind, [p[0] for p in pre] + [d[0] for d in dec], [p[1] for p in pre], [False] * len(pre),
+                     want=[p[2] for p in pre] + [d[1] for d in dec])
+
+    def update_forced(self, batch: Batch, end: list[str]) -> None:
+        """After a forced batch ran: its tokens are in the cache; requests in
+        `end` are finished and give their pages back."""
+        for r in batch.requests:
+            r.num_computed = r.num_tokens
+            self.kv.register_filled(r)
+        for rid in end:
+            r = self.forced.pop(rid, None)
+            if r is None:
+                raise KeyError(f"{rid}: not a live forced request")
+            self._finish(r, FinishReason.STOP)
 
     # ------------------------------------------------------------------ asynchronous scheduling
     def pre_update(self, batch: Batch) -> None:

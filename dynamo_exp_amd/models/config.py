@@ -131,6 +131,107 @@ class ModelConfig:
             json.dump(d, f, indent=2)
 
 
+@dataclass
+class LayeredConfig:
+    """A model given as an explicit list of layers (config.json key `layers`),
+    each naming its mixer type, the mixer's sizes and constants, and its
+    feed-forward (or none), with an optional `loop` that repeats a span of
+    layers with shared weights and per-pass caches, and optional parallel
+    residual streams.  Every size and constant comes from the file; the
+    engine-facing fields below mirror ModelConfig's."""
+
+    name: str = "layered"
+    architecture: str = "Bekulix"
+    vocab_size: int = 0
+    hidden_size: int = 0
+    layers: list = field(default_factory=list)  # [{"type", "mixer": {...}, "mlp": {...} | None}]
+    loop: dict | None = None  # {"start", "stop", "times"}
+    rms_norm_eps: float = 1e-6
+    streams: int | None = None  # parallel residual streams (None: one plain residual)
+    max_position_embeddings: int = 1 << 20
+    tie_word_embeddings: bool = False
+    bos_token_id: int = 0
+    eos_token_id: list[int] = field(default_factory=list)
+    vision: dict | None = None
+    image_token_id: int | None = None
+
+    def layer_runs(self) -> list[int]:
+        """Layer index of every layer run, in execution order."""
+        n = len(self.layers)
+        lp = self.loop
+        if not lp:
+            return list(range(n))
+        a, b, times = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+        if not (0 <= a <= b <= n and times >= 1):
+            raise ValueError(f"bad loop {lp!r} for {n} layers")
+        return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layer_runs())
+
+    def num_params(self) -> int:
+        W = self.hidden_size
+        n = 2 * self.vocab_size * W + W
+        for L in self.layers:
+            m, t = L["mixer"], L["type"]
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            if t == "latent_attention":
+                r = m["kv_rank"]
+                n += H * d * W + r * W + H * d * r + H * dv * r + W * H * dv
+            elif t == "attention":
+                n += (H + m["kv_heads"]) * d * W + W * H * dv
+            else:
+                n += (2 * H * d + 2 * m["kv_heads"] * d + m["kv_heads"] * dv) * W + W * H * dv
+            if L.get("mlp"):
+                n += 3 * W * L["mlp"]["ff"]
+        return n
+
+    def to_dict(self) -> dict:
+        return dataclasses.asdict(self)
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "layered") -> "LayeredConfig":
+        """From the checkpoint's config.json."""
+        return cls(name=name, architecture=c["architecture"], vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                   layers=list(c["layers"]), loop=c.get("loop"), rms_norm_eps=float(c["norm"]["eps"]),
+                   streams=c.get("streams"),
+                   max_position_embeddings=int(c.get("max_position_embeddings", 1 << 20)),
+                   eos_token_id=list(c.get("eos_token_id", [])))
+
+    def write_hf_config(self, path: str) -> None:
+        os.makedirs(path, exist_ok=True)
+        d = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+             "layers": self.layers, "norm": {"eps": self.rms_norm_eps}}
+        if self.loop:
+            d["loop"] = self.loop
+        if self.streams:
+            d["streams"] = self.streams
+        with open(os.path.join(path, "config.json"), "w") as f:
+            json.dump(d, f, indent=1)
+
+
+# config.json `architecture` values served by LayeredConfig
+LAYERED_ARCHITECTURES = ("Bekulix",)
+
+
+def _bekulix_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, window, chunk, vocab=32000, streams=4):
+    """A Bekulix stack at a real model's layer sizes: latent (windowed), plain
+    and differential (chunked) attention layers in turn."""
+    att = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d,
+                                          "scale": d ** -0.5, "q_temp": {"coef": 0.1, "every": 4096}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    lat = {"type": "latent_attention", "mixer": {"heads": heads, "dim": d, "vdim": d, "kv_rank": rank,
+                                                 "scale": d ** -0.5, "mask": {"size": window}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    dif = {"type": "attention_2", "mixer": {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": d,
+                                            "vdim": 2 * d, "scale": d ** -0.5, "diff": 0.8, "mask": {"size": chunk}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    cyc = [att, lat, att, dif]
+    return LayeredConfig(name=name, vocab_size=vocab, hidden_size=W, layers=[dict(cyc[i % 4]) for i in range(n_layers)],
+                         streams=streams)
+
+
 # CLIP ViT-L/14 at 336 px, the LLaVA-1.5 vision tower; features from the
 # second-to-last layer, CLS dropped, projected by a 2-layer GELU MLP
 CLIP_L_336 = {
@@ -183,6 +284,12 @@ PRESETS: dict[str, ModelConfig] = {
 }
 
 
+PRESETS["bekulix-tiny"] = _bekulix_preset("bekulix-tiny", 256, 512, 4, 4, 2, 64, 64, 48, 96, vocab=512)
+# Llama-3-8B's layer sizes (width 4096, ff 14336, 32 x 128 heads, 8 KV heads), 8 layers
+PRESETS["bekulix-8b-shapes"] = _bekulix_preset("bekulix-8b-shapes", 4096, 14336, 8, 32, 8, 128, 512, 1024, 2048,
+                                               vocab=128256)
+
+
 def get_config(name_or_path: str) -> ModelConfig:
     """A preset, an HF directory, or `<preset>@<layers>`: the preset's
     architecture truncated to its first <layers> decoder layers (one-GPU
@@ -199,6 +306,10 @@ def get_config(name_or_path: str) -> ModelConfig:
     if name_or_path in PRESETS:
         return dataclasses.replace(PRESETS[name_or_path])
     if os.path.isdir(name_or_path) and os.path.exists(os.path.join(name_or_path, "config.json")):
+        with open(os.path.join(name_or_path, "config.json")) as f:
+            raw = json.load(f)
+        if raw.get("architecture") in LAYERED_ARCHITECTURES:  # the model class follows the file
+            return LayeredConfig.from_dict(raw, name=os.path.basename(os.path.normpath(name_or_path)))
         return ModelConfig.from_hf_dir(name_or_path)
     key = name_or_path.lower().replace("meta-llama/", "").replace("meta-", "")
     for k in PRESETS:

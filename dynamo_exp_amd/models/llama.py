@@ -60,6 +60,13 @@ class AttnMeta:
     # multimodal: rows of the token stream whose embeddings are replaced
     mm_rows: torch.Tensor | None = None
     mm_embeds: torch.Tensor | None = None
+    # models with `unified_rows` (one attention launch over prompt-chunk and
+    # decode rows alike): every row's sequence, as a row of row_tables, which
+    # stacks the block tables of the prefill and the decode requests
+    row_seq: torch.Tensor | None = None  # [T] int32
+    row_tables: torch.Tensor | None = None  # [n_prefill + n_decode, max_blocks] int32
+    block_size: int = 0
+    max_ctx: int = 0  # longest context of the step known on the host (0: unknown)
 
 
 class TPGroup:
@@ -769,10 +776,11 @@ class LlamaForCausalLM:
             self._side = streams.stream("side", self.device)  # high priority: utils/streams.py
         return self._side
 
-    def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        """Full-vocab logits (all-gathered over TP ranks)."""
+    def compute_logits(self, hidden: torch.Tensor, fp32: bool = False) -> torch.Tensor:
+        """Full-vocab logits (all-gathered over TP ranks); fp32: as float32 (scoring)."""
         logits = self._mm(hidden, self.lm_head)
-        return self.tp.all_gather_last(logits)
+        logits = self.tp.all_gather_last(logits)
+        return logits.float() if fp32 else logits
 
     def sample_sharded(self, hidden: torch.Tensor, temperature, seeds, offsets, out_tokens=None, out_logprobs=None):
         """Greedy / temperature sampling without gathering the logits: every

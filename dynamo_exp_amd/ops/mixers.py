@@ -1,0 +1,268 @@
+"""Ops of the layer-listed (hybrid) models: multi-stream residual steps, gated
+feed-forward activations, per-head q/k preparation fused with the paged cache
+write, masked paged attention over rows of mixed sequences, and the two-map
+(differential) combine.
+
+GPU tensors run the gfx950 kernels of ``_C_mixers`` (csrc/mixers); CPU tensors
+run the PyTorch forms below (CPU CI of the engine).  A GPU call never falls
+back.  Every op works on bf16 or fp32 activations; residual streams, norms,
+scores and softmax weights are fp32 in both.
+
+Layouts:
+  * residual streams X [T, S, W] fp32, updated in place
+  * paged caches, token-major: K [num_blocks * block_size, Wk], V likewise
+    [.., Wv]; slot = block * block_size + offset
+  * rows of one step: positions [T] int64, slots [T] int64 (-1: not cached),
+    seq [T] int32 -> row of block_tables (None: row i is sequence i)
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import _native
+
+MASKS = {"causal": 0, "window": 1, "chunk": 2}
+ACTS = {"relu": 0, "silu": 1, "gelu_tanh": 2}
+MAX_STREAMS = 8
+# row attention: aim for this many waves per launch, never split a row's keys
+# into parts shorter than ROW_MIN_PART
+ROW_TARGET_WAVES = 2048
+ROW_MIN_PART = 256
+
+
+def _m():
+    return _native.mixers()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _f32(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return 1
+    if t.dtype == torch.bfloat16:
+        return 0
+    raise TypeError(f"activations must be bfloat16 or float32, got {t.dtype}")
+
+
+def _ptr(t: torch.Tensor | None) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _fp32_param(t: torch.Tensor | None, name: str):
+    if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+        raise TypeError(f"{name}: expected a contiguous float32 tensor")
+
+
+# ----------------------------------------------------------------- residual streams
+def embed_streams(ids: torch.Tensor, table: torch.Tensor, n_streams: int) -> torch.Tensor:
+    """X [T, S, W] fp32 with every stream equal to table[ids]."""
+    T = ids.shape[0]
+    V, W = table.shape
+    if not table.is_cuda:
+        return table[ids].float()[:, None, :].repeat(1, n_streams, 1).contiguous()
+    X = torch.empty((T, n_streams, W), dtype=torch.float32, device=table.device)
+    ids = ids if ids.dtype == torch.int64 else ids.long()
+    _m().embed_streams(X.data_ptr(), table.data_ptr(), ids.data_ptr(), T, n_streams, W, V, _f32(table), _stream())
+    return X
+
+
+def stream_step(X: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, gain: torch.Tensor | None,
+                rin: torch.Tensor | None, norm_w: torch.Tensor | None, eps: float,
+                out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor | None:
+    """One residual step over S streams, in place on X [T, S, W] (fp32):
+    with y [T, W]:  X_t <- sum_s mix[s, t] X_s + gain[t] y   (all t from the old X);
+    with rin [S]:   returns norm(sum_s rin[s] X_s) * norm_w  (norm_w None: the plain sum).
+    S = 1 with mix = gain = rin = 1 is the ordinary pre-norm residual."""
+    T, S, W = X.shape
+    if X.dtype != torch.float32 or not X.is_contiguous():
+        raise TypeError("residual streams must be contiguous float32")
+    if S > MAX_STREAMS:
+        raise ValueError(f"{S} residual streams (kernel limit {MAX_STREAMS})")
+    for t, n in ((mix, "mix"), (gain, "gain"), (rin, "rin"), (norm_w, "norm_w")):
+        _fp32_param(t, n)
+    if not X.is_cuda:
+        if y is not None:
+            X.copy_(torch.einsum("st,nsw->ntw", mix, X) + gain[None, :, None] * y.float()[:, None, :])
+        if rin is None:
+            return None
+        u = torch.einsum("s,nsw->nw", rin, X)
+        if norm_w is not None:
+            u = u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * norm_w
+        return u.to(out_dtype)
+    out = torch.empty((T, W), dtype=out_dtype, device=X.device) if rin is not None else None
+    if y is not None:
+        if y.dtype != out_dtype and out is not None:
+            raise TypeError("y and the output share one activation dtype")
+        if y.stride(-1) != 1:
+            raise ValueError("y: last dim must be contiguous")
+    f32 = _f32(y) if y is not None else int(out_dtype == torch.float32)
+    _m().stream_step(X.data_ptr(), _ptr(y), y.stride(0) if y is not None else 0, _ptr(mix), _ptr(gain), _ptr(rin),
+                     _ptr(norm_w), float(eps), _ptr(out), W, T, S, W, f32, _stream())
+    return out
+
+
+# ----------------------------------------------------------------- feed-forward
+def _act(z: torch.Tensor, act: str) -> torch.Tensor:
+    if act == "relu":
+        return torch.relu(z)
+    if act == "silu":
+        return z * torch.sigmoid(z)
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def glu_act(gu: torch.Tensor, act: str = "relu") -> torch.Tensor:
+    """[T, 2F] = [gate | up] -> act(gate) * up, [T, F]."""
+    T, F2 = gu.shape
+    F = F2 // 2
+    if act not in ACTS:
+        raise ValueError(f"unknown activation {act!r}")
+    if not gu.is_cuda:
+        g, u = gu.float().split(F, dim=1)
+        return (_act(g, act) * u).to(gu.dtype)
+    out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
+    _m().glu_act(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0), F, ACTS[act], _f32(gu), _stream())
+    return out
+
+
+# ----------------------------------------------------------------- q/k preparation + cache write
+def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, n_q: int, n_k: int, d: int,
+                   k_off: int, q_w: torch.Tensor | None, k_w: torch.Tensor | None, eps: float,
+                   temp: tuple[float, float] | None, kc: torch.Tensor, vc: torch.Tensor | None, v_mode: int = 0,
+                   v_off: int = 0, v_w: int = 0) -> None:
+    """Per row of the fused projection output x = [q | k | v] (in place):
+    q heads: unit RMS times q_w (when given) and the position gain
+    1 + coef * ln(floor((p + 1) / every) + 1) (temp = (coef, every));
+    k heads at column k_off: unit RMS times k_w (when given) into the K cache;
+    v_mode 0: no V cache; 1: the k columns as projected are the value;
+    2: the v_w columns at v_off are.  Rows with slot < 0 cache nothing."""
+    T = x.shape[0]
+    coef, every = (float(temp[0]), float(temp[1])) if temp else (0.0, 1.0)
+    _fp32_param(q_w, "q_w")
+    _fp32_param(k_w, "k_w")
+    if x.stride(-1) != 1 or kc.dtype != x.dtype or not kc.is_contiguous():
+        raise ValueError("headprep_cache: x rows contiguous, caches contiguous and of x's dtype")
+    k_wd = n_k * d
+    if kc.shape[-1] != k_wd or (v_mode == 1 and vc.shape[-1] != k_wd) or (v_mode == 2 and vc.shape[-1] != v_w):
+        raise ValueError("headprep_cache: cache row widths do not match the sections")
+    if max(n_q * d, k_off + k_wd, (v_off + v_w) if v_mode == 2 else 0) > x.shape[1]:
+        raise ValueError("headprep_cache: sections exceed the row")
+    if not x.is_cuda:
+        xf = x.float()
+        if q_w is not None or coef != 0.0:
+            q = xf[:, : n_q * d].reshape(T, n_q, d)
+            if q_w is not None:
+                q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_w
+            if coef != 0.0:
+                k_ = torch.floor((positions.double() + 1.0) / every).float()
+                q = q * (1.0 + coef * torch.log(k_ + 1.0))[:, None, None]
+            x[:, : n_q * d] = q.reshape(T, n_q * d).to(x.dtype)
+        ok = slots >= 0
+        sl = slots[ok]
+        k = xf[ok, k_off:k_off + k_wd]
+        if v_mode == 1:
+            vc[sl] = x[ok, k_off:k_off + k_wd]
+        if k_w is not None:
+            kh = k.reshape(-1, n_k, d)
+            k = (kh * torch.rsqrt((kh * kh).mean(-1, keepdim=True) + eps) * k_w).reshape(-1, k_wd)
+        kc[sl] = k.to(kc.dtype)
+        if v_mode == 2:
+            vc[sl] = x[ok, v_off:v_off + v_w]
+        return
+    if positions.dtype != torch.int64 or slots.dtype != torch.int64:
+        raise TypeError("positions and slots must be int64")
+    _m().headprep_cache(x.data_ptr(), x.stride(0), positions.data_ptr(), slots.data_ptr(), T, n_q, n_k, d, k_off,
+                        _ptr(q_w), _ptr(k_w), float(eps), coef, every, kc.data_ptr(), _ptr(vc) if v_mode else 0,
+                        v_mode, v_off, v_w, _f32(x), _stream())
+
+
+# ----------------------------------------------------------------- attention
+def row_attention_parts(rows: int, n_qh: int, max_visible: int) -> int:
+    """Key partitions per row so a launch has about ROW_TARGET_WAVES waves."""
+    if rows <= 0:
+        return 1
+    want = -(-ROW_TARGET_WAVES // (rows * n_qh))
+    return max(1, min(want, max_visible // ROW_MIN_PART))
+
+
+def first_visible(p: torch.Tensor, mask: str, size: int) -> torch.Tensor:
+    if mask == "window":
+        return (p - size + 1).clamp_min(0)
+    if mask == "chunk":
+        return torch.div(p, size, rounding_mode="floor") * size
+    return torch.zeros_like(p)
+
+
+def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
+                  seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
+                  group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
+                  out_f32: bool = False) -> torch.Tensor:
+    """Softmax attention of T rows over their sequences' paged caches.
+    q [T, >= n_qh * d] (n_qh = heads * maps query vectors per row); returns
+    [T, n_qh, dv].  Query vector qh reads K head (qh // maps // group) * maps +
+    qh % maps and V head qh // maps // group."""
+    T = q.shape[0]
+    if mask not in MASKS:
+        raise ValueError(f"unknown mask {mask!r}")
+    if mask != "causal" and size < 1:
+        raise ValueError("window / chunk masks need a size >= 1")
+    if n_qh % maps or (n_qh // maps) % group:
+        raise ValueError("head counts do not divide")
+    n_kh = n_qh // maps // group * maps
+    Wk, Wv = kc.shape[-1], vc.shape[-1]
+    if Wk < n_kh * d or Wv < n_qh // maps // group * dv or q.shape[1] < n_qh * d:
+        raise ValueError("row_attention: widths do not cover the heads")
+    odt = torch.float32 if (out_f32 or q.dtype == torch.float32) else q.dtype
+    if not q.is_cuda:
+        out = torch.empty((T, n_qh, dv), dtype=torch.float32)
+        sq = seq.long() if seq is not None else torch.arange(T)
+        qf = q[:, : n_qh * d].float().reshape(T, n_qh, d)
+        heads = torch.arange(n_qh) // maps
+        kh = heads // group * maps + torch.arange(n_qh) % maps
+        vh = heads // group
+        for s in sq.unique().tolist():
+            rows = (sq == s).nonzero().flatten()
+            p = positions[rows].long()
+            n = int(p.max()) + 1
+            j = torch.arange(n)
+            sl = block_tables[s].long()[j // block_size] * block_size + j % block_size
+            K = kc[sl].float()[:, : n_kh * d].reshape(n, n_kh, d)[:, kh]  # [n, n_qh, d]
+            V = vc[sl].float()[:, : (n_qh // maps // group) * dv].reshape(n, -1, dv)[:, vh]
+            sc = torch.einsum("ihd,jhd->hij", qf[rows], K) * scale
+            vis = (j[None, :] <= p[:, None]) & (j[None, :] >= first_visible(p, mask, size)[:, None])
+            sc = sc.masked_fill(~vis[None], float("-inf"))
+            out[rows] = torch.einsum("hij,jhd->ihd", torch.softmax(sc, -1), V)
+        return out.to(odt)
+    if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous():
+        raise TypeError("row_attention: caches contiguous and of q's dtype")
+    if q.stride(1) != 1 or positions.dtype != torch.int64 or block_tables.dtype != torch.int32 or \
+            (seq is not None and seq.dtype != torch.int32) or block_tables.stride(1) != 1:
+        raise TypeError("row_attention: q rows contiguous, positions int64, seq / block_tables int32")
+    if seq is None and block_tables.shape[0] < T:
+        raise ValueError("row_attention: fewer block-table rows than rows")
+    out = torch.empty((T, n_qh, dv), dtype=odt, device=q.device)
+    ws = torch.empty((T, n_qh, parts, 2 + dv), dtype=torch.float32, device=q.device) if parts > 1 else None
+    _m().row_attention(out.data_ptr(), _ptr(ws), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
+                       positions.data_ptr(), _ptr(seq), block_tables.data_ptr(), block_tables.stride(0), block_size,
+                       T, n_qh, maps, group, d, dv, Wk, Wv, float(scale), MASKS[mask], int(size), parts, _f32(q),
+                       int(odt == torch.float32), _stream())
+    return out
+
+
+def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a [T, H, 2, dv] fp32 (two maps' outputs) -> [T, H * dv]:
+    unit_rms_over_dv(a1 - lam * a2) * post."""
+    T, H, two, dv = a.shape
+    if two != 2 or a.dtype != torch.float32 or not a.is_contiguous():
+        raise TypeError("diff_combine: a must be contiguous float32 [T, H, 2, dv]")
+    if not a.is_cuda:
+        o = a[:, :, 0] - lam * a[:, :, 1]
+        o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * post
+        return o.reshape(T, H * dv).to(out_dtype)
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=a.device)
+    _m().diff_combine(out.data_ptr(), a.data_ptr(), T * H, dv, float(lam), float(post), float(eps),
+                      int(out_dtype == torch.float32), _stream())
+    return out
