@@ -24,6 +24,9 @@ int dxm_diff_combine(void*, const float*, int64_t, int, float, float, float, int
 int dxm_row_attention(void*, float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*,
                       const int*, int, int, int, int, int, int, int, int, int, int, float, int, int, int, int, int,
                       hipStream_t);
+int dxm_tile_attention_ok(int, int);
+int dxm_tile_attention(void*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*,
+                       int, int, const int*, int, int, int, int, int, int, int, int, float, int, int, int, hipStream_t);
 }
 
 static void check(int rc, const char* what) {
@@ -59,6 +62,16 @@ PYBIND11_MODULE(_C_mixers, m) {
   });
   m.def("diff_combine", [](u out, u a, int64_t n_vec, int dv, float lam, float post, float eps, int f32, u st) {
     check(dxm_diff_combine(P(out), F(a), n_vec, dv, lam, post, eps, f32, S(st)), "diff_combine");
+  });
+  m.def("tile_attention_ok", &dxm_tile_attention_ok);
+  m.def("tile_attention", [](u out, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, u tiles,
+                             int n_tiles, int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale,
+                             int mask, int size, int out_f32, u st) {
+    check(dxm_tile_attention(P(out), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
+                             reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs,
+                             reinterpret_cast<const int*>(tiles), n_tiles, n_qh, maps, group, d, dv, Wk, Wv, scale,
+                             mask, size, out_f32, S(st)),
+          "tile_attention");
   });
   m.def("row_attention", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                             int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,

@@ -1,0 +1,261 @@
+// Paged softmax attention for prompt chunks on the gfx950 matrix cores: the
+// prefill kernel of the layer-listed models (bf16 q / caches, head widths that
+// are multiples of 16; everything else runs row_attention.hip).
+//
+// A workgroup (4 waves) takes up to 128 consecutive rows of one sequence and
+// one query vector (head x map); a wave owns 32 of the rows as two 16-row
+// blocks.  64-key tiles of the paged, token-major caches are staged in LDS (K
+// row-major, V transposed) and shared by the four waves.  Both products are
+// "swapped" so the query sits on the lane:
+//     S^T = K Q^T     A = K rows (LDS), B = Q^T (registers, loaded once)
+//     O^T = V^T P^T   A = V^T (LDS),    B = P^T = the S^T accumulator itself
+// (v_mfma_f32_16x16x16_bf16: lane l holds column l % 16 and rows 4 (l / 16)
+// .. + 3 of C, which is exactly the B layout of the next product).  Scores are
+// the exact fp32 sums of bf16 products; the softmax is fp32; the weights enter
+// the second product as a bf16 pair hi + lo (two MFMAs), which keeps 16
+// mantissa bits of every weight instead of 8.
+//
+// Masks are evaluated per element in sequence positions: causal, sliding
+// window (p - size < j <= p) and chunked (floor(j / size) == floor(p / size)),
+// so a prompt cut anywhere gives the same result as one cut nowhere.
+#include "../kernels/common.h"
+
+namespace {
+
+constexpr int kRows = 128;  // rows per workgroup
+constexpr int kKeys = 64;   // keys per tile
+constexpr int kVtStride = kKeys + 8;
+
+struct TileArgs {
+  const bf16_t* q;
+  int64_t q_stride;
+  const bf16_t* kc;
+  const bf16_t* vc;
+  void* out;  // [rows, n_qh, dv]
+  const int64_t* pos;
+  const int* seq;
+  const int* bt;
+  int bt_stride, bs;
+  const int* tiles;  // [n_tiles, 2]: first row, row count (<= 128; one sequence, consecutive positions)
+  int n_qh, maps, group;
+  int Wk, Wv;
+  float scale;
+  int mask, size;
+};
+
+__device__ __forceinline__ int64_t first_visible(int64_t p, int mask, int size) {
+  if (mask == 1) return p - size + 1 > 0 ? p - size + 1 : 0;
+  if (mask == 2) return p / size * size;
+  return 0;
+}
+
+template <typename OutT> __device__ __forceinline__ void store4(OutT* o, f32x4 v);
+template <> __device__ __forceinline__ void store4<float>(float* o, f32x4 v) { *reinterpret_cast<f32x4*>(o) = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* o, f32x4 v) {
+  uint2 w;
+  w.x = pack_bf16x2(v[0], v[1]);
+  w.y = pack_bf16x2(v[2], v[3]);
+  *reinterpret_cast<uint2*>(o) = w;
+}
+
+template <int DB, int DVB, typename OutT>
+__global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
+  constexpr int d = DB * 16, dv = DVB * 16, ks_stride = d + 8;
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+  bf16_t* Ks = smem;                    // [64][d + 8]
+  bf16_t* Vt = smem + kKeys * ks_stride;  // [dv][64 + 8]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int c16 = lane & 15, g4 = lane >> 4;
+  const int qh = blockIdx.x;
+  const int row0 = a.tiles[2 * blockIdx.y], n = a.tiles[2 * blockIdx.y + 1];
+  const int64_t p0 = a.pos[row0];
+  const int* bt = a.bt + (int64_t)a.seq[row0] * a.bt_stride;
+  const int head = qh / a.maps, m = qh - head * a.maps, g = head / a.group;
+  const bf16_t* kc = a.kc + (int64_t)(g * a.maps + m) * d;
+  const bf16_t* vc = a.vc + (int64_t)g * dv;
+  const int64_t hi = p0 + n - 1;
+  const int64_t kt0 = first_visible(p0, a.mask, a.size) / kKeys * kKeys;
+
+  // this wave's query fragments and per-row constants
+  i16x4 qf[2][DB];
+  int64_t prow[2], lrow[2];
+  bool okrow[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int r = 32 * w + 16 * qb + c16;
+    okrow[qb] = r < n;
+    prow[qb] = p0 + r;
+    lrow[qb] = first_visible(prow[qb], a.mask, a.size);
+    const bf16_t* q = a.q + (int64_t)(row0 + (okrow[qb] ? r : 0)) * a.q_stride + (int64_t)qh * d + 4 * g4;
+#pragma unroll
+    for (int ks = 0; ks < DB; ++ks)
+      qf[qb][ks] = okrow[qb] ? *reinterpret_cast<const i16x4*>(q + ks * 16) : i16x4{0, 0, 0, 0};
+  }
+  const bool wave_on = 32 * w < n;
+  float mx[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
+  f32x4 O[2][DVB];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int64_t kt = kt0; kt <= hi; kt += kKeys) {
+    {  // stage the tile: 4 threads per key
+      const int key = tid >> 2, part = tid & 3;
+      const int64_t kj = kt + key;
+      const bool ok = kj <= hi;
+      const int64_t slot = ok ? (int64_t)bt[kj / a.bs] * a.bs + kj % a.bs : 0;
+      const bf16_t* ksrc = kc + slot * a.Wk;
+      const bf16_t* vsrc = vc + slot * a.Wv;
+      const u16x8 zero = {{0, 0, 0, 0}};
+      for (int c = part * 8; c < d; c += 32)
+        *reinterpret_cast<u16x8*>(Ks + key * ks_stride + c) = ok ? *reinterpret_cast<const u16x8*>(ksrc + c) : zero;
+      for (int c = part * 8; c < dv; c += 32) {
+        const u16x8 v = ok ? *reinterpret_cast<const u16x8*>(vsrc + c) : zero;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          Vt[(c + 2 * i) * kVtStride + key] = (bf16_t)(v.w[i] & 0xffffu);
+          Vt[(c + 2 * i + 1) * kVtStride + key] = (bf16_t)(v.w[i] >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    if (wave_on) {
+      f32x4 S[2][4];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        S[0][kb] = S[1][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < DB; ++ks) {
+          const i16x4 A = *reinterpret_cast<const i16x4*>(Ks + (kb * 16 + c16) * ks_stride + ks * 16 + 4 * g4);
+          S[0][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[0][ks], S[0][kb], 0, 0, 0);
+          S[1][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[1][ks], S[1][kb], 0, 0, 0);
+        }
+      }
+      i16x4 Ph[2][4], Pl[2][4];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int64_t kj = kt + kb * 16 + 4 * g4 + i;
+            const bool vis = okrow[qb] && kj >= lrow[qb] && kj <= prow[qb];
+            const float s = vis ? S[qb][kb][i] * a.scale : -INFINITY;
+            S[qb][kb][i] = s;
+            mloc = fmaxf(mloc, s);
+          }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+        const float mn = fmaxf(mx[qb], mloc);
+        const float mu = mn == -INFINITY ? 0.f : mn;  // a row that sees nothing in this tile
+        const float alpha = __expf(mx[qb] - mu);
+        mx[qb] = mn;
+        float add = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+          float p[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            p[i] = __expf(S[qb][kb][i] - mu);
+            add += p[i];
+          }
+          const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
+          const uint32_t l01 = pack_bf16x2(p[0] - bf16lo(h01), p[1] - bf16hi(h01));
+          const uint32_t l23 = pack_bf16x2(p[2] - bf16lo(h23), p[3] - bf16hi(h23));
+          Ph[qb][kb] = __builtin_bit_cast(i16x4, uint2{h01, h23});
+          Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
+        }
+        lsum[qb] = lsum[qb] * alpha + add;
+#pragma unroll
+        for (int cb = 0; cb < DVB; ++cb) O[qb][cb] *= alpha;
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int cb = 0; cb < DVB; ++cb) {
+          const i16x4 A = *reinterpret_cast<const i16x4*>(Vt + (cb * 16 + c16) * kVtStride + kb * 16 + 4 * g4);
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb) {
+            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Ph[qb][kb], O[qb][cb], 0, 0, 0);
+            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Pl[qb][kb], O[qb][cb], 0, 0, 0);
+          }
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    float l = lsum[qb];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!okrow[qb]) continue;
+    const float inv = 1.f / l;
+    const int r = 32 * w + 16 * qb + c16;
+    OutT* o = (OutT*)a.out + ((int64_t)(row0 + r) * a.n_qh + qh) * dv + 4 * g4;
+#pragma unroll
+    for (int cb = 0; cb < DVB; ++cb) store4<OutT>(o + cb * 16, O[qb][cb] * inv);
+  }
+}
+
+template <int DB, int DVB, typename OutT>
+int launch_tiles(const TileArgs& a, int n_tiles, hipStream_t st) {
+  const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * kVtStride) * sizeof(bf16_t);
+  auto kern = tile_attention_kernel<DB, DVB, OutT>;
+  if (lds > 48 * 1024) {
+    static bool raised = false;  // per instantiation
+    if (!raised) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return 7;
+      raised = true;
+    }
+  }
+  for (int t0 = 0; t0 < n_tiles; t0 += 65535) {
+    TileArgs b = a;
+    b.tiles = a.tiles + 2 * t0;
+    const int nt = n_tiles - t0 < 65535 ? n_tiles - t0 : 65535;
+    hipLaunchKernelGGL(kern, dim3(a.n_qh, nt), dim3(256), lds, st, b);
+  }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+}  // namespace
+
+#define TILE_CASE(DB_, DVB_)                                                               \
+  if (d == DB_ * 16 && dv == DVB_ * 16)                                                    \
+    return out_f32 ? launch_tiles<DB_, DVB_, float>(a, n_tiles, st) : launch_tiles<DB_, DVB_, bf16_t>(a, n_tiles, st);
+
+extern "C" {
+
+// 1 when tile_attention has an instance for the head widths
+int dxm_tile_attention_ok(int d, int dv) {
+  const int pairs[][2] = {{2, 2}, {3, 3}, {3, 6}, {4, 4}, {4, 8}, {8, 8}, {8, 16}, {16, 16}};
+  for (auto& p : pairs)
+    if (d == p[0] * 16 && dv == p[1] * 16) return 1;
+  return 0;
+}
+
+int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
+                       const int* seq, const int* bt, int bt_stride, int bs, const int* tiles, int n_tiles, int n_qh,
+                       int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask, int size, int out_f32,
+                       hipStream_t st) {
+  if (n_tiles <= 0) return 0;
+  if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
+  if (mask < 0 || mask > 2 || (mask && size < 1)) return 3;
+  if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
+  TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
+             tiles, n_qh, maps, group, Wk, Wv, scale, mask, size};
+  TILE_CASE(2, 2)
+  TILE_CASE(3, 3)
+  TILE_CASE(3, 6)
+  TILE_CASE(4, 4)
+  TILE_CASE(4, 8)
+  TILE_CASE(8, 8)
+  TILE_CASE(8, 16)
+  TILE_CASE(16, 16)
+  return 2;
+}
+
+}  // extern "C"

@@ -24,6 +24,7 @@ import numpy as np
 import torch
 
 from .. import ops
+from ..ops import mixers as mixer_ops
 from ..models.llama import AttnMeta, LlamaForCausalLM  # noqa: F401 -- any registered model class fits
 from .request import Request
 
@@ -255,6 +256,8 @@ class ModelRunner:
             num_prefill_tokens=cu[-1],
             row_seq=self._to_dev(seq, torch.int32),
             row_tables=self._to_dev(self._block_table(allr), torch.int32),
+            row_tiles=self._to_dev(np.asarray([t for c, n in zip(cu, num_new) for t in mixer_ops.tile_list(c, n)],
+                                              dtype=np.int32).reshape(-1, 2), torch.int32) if reqs else None,
             block_size=self.block_size,
             max_ctx=max(ctx) if ctx else 0,
         )

@@ -10,7 +10,9 @@ chunks and decode tokens of different sequences side by side):
                                                  fp32 streams, read in, RMS norm (1 + w)
     p  = h @ Wfused^T (+ b)                 hipBLASLt, one fused projection per mixer
     headprep_cache(p)                       HIP  q/k head norms, position gain, paged cache write
-    a  = row_attention(q, K cache, V cache) HIP  causal / sliding-window / chunked masks
+    a  = attention(q, K cache, V cache)     HIP  causal / sliding-window / chunked masks; prompt
+                                                 chunks on the MFMA tile kernel, decode rows (and
+                                                 fp32, odd head widths) on the row kernel
     [a = diff_combine(a)]                   HIP  two-map (differential) layers
     y  = a @ Wo^T                           hipBLASLt
     h  = stream_step(X, y)                  HIP
@@ -272,14 +274,16 @@ class BekulixForCausalLM:
         m, T = L["m"], h.shape[0]
         H, d, eps = m["heads"], m["dim"], self.cfg.rms_norm_eps
         pos, slots = meta.positions, meta.slot_mapping
+        # prompt-chunk rows (the first num_prefill_tokens) as tiles for the matrix-core kernel
+        tl = (meta.row_tiles, meta.num_prefill_tokens) if meta.is_prefill else (None, 0)
         if L["type"] == "attention":
             G = m["kv_heads"]
             p = torch.matmul(h, L["w_in"].t())
             qt = m.get("q_temp")
             mx.headprep_cache(p, pos, slots, H, G, d, H * d, L["qn"], L["kn"], eps,
                               (qt["coef"], qt["every"]) if qt else None, kc, vc, v_mode=1)
-            a = mx.row_attention(p, kc, vc, pos, seq, tables, bs, H, 1, H // G, d, d, m["scale"], "causal", 0,
-                                 self._parts(T, H, "causal", 0, meta))
+            a = mx.attention(p, kc, vc, pos, seq, tables, bs, H, 1, H // G, d, d, m["scale"], "causal", 0,
+                             self._parts(T, H, "causal", 0, meta), False, *tl)
             return torch.matmul(a.view(T, H * d), L["w_o"].t())
         if L["type"] == "latent_attention":
             r, dv, size = m["kv_rank"], m["vdim"], m["mask"]["size"]
@@ -287,8 +291,8 @@ class BekulixForCausalLM:
             mx.headprep_cache(p, pos, slots, 0, 1, r, H * d, None, L["cn"], eps, None, kc, None, v_mode=0)
             # fold W_uk into the query: the latent cache is the one key/value head of every query head
             ql = torch.bmm(p[:, : H * d].view(T, H, d).transpose(0, 1), L["uk"]).transpose(0, 1).contiguous()
-            a = mx.row_attention(ql.view(T, H * r), kc, kc, pos, seq, tables, bs, H, 1, H, r, r, m["scale"], "window",
-                                 size, self._parts(T, H, "window", size, meta))
+            a = mx.attention(ql.view(T, H * r), kc, kc, pos, seq, tables, bs, H, 1, H, r, r, m["scale"], "window",
+                             size, self._parts(T, H, "window", size, meta), False, *tl)
             o = torch.bmm(a.transpose(0, 1), L["uv"]).transpose(0, 1).reshape(T, H * dv)
             return torch.matmul(o, L["w_o"].t())
         G, dv, size = m["kv_heads"], m["vdim"], m["mask"]["size"]
@@ -296,8 +300,8 @@ class BekulixForCausalLM:
         qw, kw = H * 2 * d, G * 2 * d
         mx.headprep_cache(p, pos, slots, 0, 2 * G, d, qw, None, None, eps, None, kc, vc, v_mode=2, v_off=qw + kw,
                           v_w=G * dv)
-        a = mx.row_attention(p, kc, vc, pos, seq, tables, bs, 2 * H, 2, H // G, d, dv, m["scale"], "chunk", size,
-                             self._parts(T, 2 * H, "chunk", size, meta), out_f32=True)
+        a = mx.attention(p, kc, vc, pos, seq, tables, bs, 2 * H, 2, H // G, d, dv, m["scale"], "chunk", size,
+                         self._parts(T, 2 * H, "chunk", size, meta), True, *tl)
         o = mx.diff_combine(a.view(T, H, 2, dv), L["lam"], 1.0 - float(m["diff"]), eps, self.dtype)
         return torch.matmul(o, L["w_o"].t())
 

@@ -65,6 +65,7 @@ class AttnMeta:
     # stacks the block tables of the prefill and the decode requests
     row_seq: torch.Tensor | None = None  # [T] int32
     row_tables: torch.Tensor | None = None  # [n_prefill + n_decode, max_blocks] int32
+    row_tiles: torch.Tensor | None = None  # [n, 2] int32: (first row, rows) tiles of the prompt-chunk rows
     block_size: int = 0
     max_ctx: int = 0  # longest context of the step known on the host (0: unknown)
 

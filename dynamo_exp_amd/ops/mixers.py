@@ -196,6 +196,52 @@ def first_visible(p: torch.Tensor, mask: str, size: int) -> torch.Tensor:
     return torch.zeros_like(p)
 
 
+TILE_ROWS = 128  # rows of one sequence per tile_attention workgroup
+
+
+def tile_list(row0: int, n: int) -> list[tuple[int, int]]:
+    """(first row, row count) tiles of a prompt chunk of n rows starting at stream row row0."""
+    return [(row0 + t, min(TILE_ROWS, n - t)) for t in range(0, n, TILE_ROWS)]
+
+
+def tile_attention_ok(q: torch.Tensor, d: int, dv: int) -> bool:
+    """Whether the matrix-core prefill kernel serves these rows (bf16 on the
+    GPU, head widths it is instantiated for); otherwise row_attention does."""
+    return q.is_cuda and q.dtype == torch.bfloat16 and bool(_m().tile_attention_ok(d, dv))
+
+
+def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
+              seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
+              group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
+              out_f32: bool = False, tiles: torch.Tensor | None = None, n_tile_rows: int = 0) -> torch.Tensor:
+    """Attention of one step's rows: the first n_tile_rows rows (prompt chunks,
+    cut into `tiles` [n, 2] = first row, row count) on the matrix-core prefill
+    kernel where it applies, all other rows (decode tokens; every row when it
+    does not apply) on the row kernel.  Same arguments and result as
+    row_attention."""
+    T = q.shape[0]
+    if tiles is None or n_tile_rows == 0 or not tile_attention_ok(q, d, dv):
+        return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
+                             mask, size, parts, out_f32)
+    if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous() or \
+            q.stride(1) != 1 or seq is None or seq.dtype != torch.int32 or positions.dtype != torch.int64 or \
+            block_tables.dtype != torch.int32 or tiles.dtype != torch.int32 or not tiles.is_contiguous():
+        raise TypeError("attention: bf16 caches, int32 seq / block_tables / tiles, int64 positions")
+    if n_qh % maps or (n_qh // maps) % group or mask not in MASKS or (mask != "causal" and size < 1):
+        raise ValueError("attention: bad head counts or mask")
+    odt = torch.float32 if out_f32 else q.dtype
+    out = torch.empty((T, n_qh, dv), dtype=odt, device=q.device)
+    _m().tile_attention(out.data_ptr(), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), positions.data_ptr(),
+                        seq.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), block_size, tiles.data_ptr(),
+                        tiles.shape[0], n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale),
+                        MASKS[mask], int(size), int(out_f32), _stream())
+    if n_tile_rows < T:
+        r = slice(n_tile_rows, T)
+        out[r] = row_attention(q[r], kc, vc, positions[r], seq[r], block_tables, block_size, n_qh, maps, group, d, dv,
+                               scale, mask, size, parts, out_f32)
+    return out
+
+
 def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
                   seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
                   group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,

@@ -70,6 +70,10 @@ CONFIGS = {
     "ones": lambda: config([att(H=4, G=1, d=8, every=1), lat(H=2, d=8, dv=8, r=8, window=1),
                             dif(H=2, G=1, d=8, dv=8, chunk=1, diff=0.0)], width=32, streams=1,
                            loop={"start": 1, "stop": 2, "times": 1}),
+    # head widths the matrix-core prefill kernel serves (bf16 on the GPU)
+    "tiles": lambda: config([att(H=4, G=2, d=32, every=16), lat(H=2, d=16, dv=32, r=48, window=20),
+                             dif(H=2, G=1, d=64, dv=128, chunk=24), att(H=2, G=1, d=64, coef=0.0)], width=64,
+                            streams=2, loop={"start": 1, "stop": 3, "times": 2}),
     # no streams at all (plain residual), heads == kv heads, wide value heads (> 64 columns)
     "plain": lambda: config([dif(H=2, G=2, d=24, dv=136, chunk=9), lat(H=3, d=8, dv=72, r=80, window=11),
                              att(H=2, G=2, d=72, every=3)], width=64, streams=None),
@@ -187,6 +191,50 @@ def test_row_attention_alone(device, mask, size, dims):
     got = mx.row_attention(qd[rows], kc, vc, pos[rows], None, table.expand(len(rows), -1).contiguous(), bs, H * maps,
                            maps, H // G, d, dv, 0.3, mask, size, parts=2)
     assert torch.allclose(got.cpu().double().view(-1, H, maps, dv), want[rows.cpu()], atol=2e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mask,size", [("causal", 0), ("window", 70), ("window", 3), ("chunk", 50), ("chunk", 200)])
+@pytest.mark.parametrize("dims", [(4, 2, 1, 32, 32), (2, 1, 2, 64, 128), (3, 3, 1, 128, 128), (2, 2, 1, 48, 48),
+                                  (2, 1, 1, 256, 256), (2, 1, 2, 128, 256), (2, 2, 2, 48, 96)])
+def test_tile_attention_alone(mask, size, dims):
+    """The matrix-core prefill kernel: a 263-row portion that starts at position
+    37 of a cached prefix (three tiles, the last ragged, cut inside pages,
+    windows and chunks) beside two decode rows of another sequence, against
+    dense masked softmax over the bf16 values; fp32 output, so the weights'
+    precision shows."""
+    H, G, maps, d, dv = dims
+    T, bs, start = 300, 16, 37
+    torch.manual_seed(5)
+    q = torch.randn(T, H, maps, d).bfloat16()
+    k = (torch.randn(T, G, maps, d) * 0.5).bfloat16()
+    v = torch.randn(T, G, dv).bfloat16()
+    vis = O.visible(T, mask, size)
+    want = torch.stack([O.softmax_attend(q[:, :, m].double(), O.expand_heads(k[:, :, m].double(), H),
+                                         O.expand_heads(v.double(), H), 0.2, vis) for m in range(maps)], 2)
+    perm = torch.randperm(40, generator=torch.Generator().manual_seed(3)).to(torch.int32)
+    table = torch.stack([perm[:19], perm[19:38]]).contiguous().cuda()  # two sequences, the same tokens on other pages
+    j = torch.arange(T, device="cuda")
+    slots, s2 = (table[i].long()[j // bs] * bs + j % bs for i in (0, 1))
+    kc = torch.zeros(40 * bs, G * maps * d, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros(40 * bs, G * dv, device="cuda", dtype=torch.bfloat16)
+    for sl in (slots, s2):
+        kc[sl] = k.reshape(T, -1).cuda()
+        vc[sl] = v.reshape(T, -1).cuda()
+    rows = list(range(start, T)) + [5, 290]
+    n_pre = T - start
+    pos = torch.tensor(rows, device="cuda")
+    seq = torch.tensor([0] * n_pre + [1, 1], dtype=torch.int32, device="cuda")
+    tiles = torch.tensor(mx.tile_list(0, n_pre), dtype=torch.int32, device="cuda")
+    qd = q.reshape(T, -1).cuda()[pos]
+    assert mx.tile_attention_ok(qd, d, dv)
+    got = mx.attention(qd, kc, vc, pos, seq, table, bs, H * maps, maps, H // G, d, dv, 0.2, mask, size, 1, True, tiles,
+                       n_pre)
+    err = (got.cpu().double().view(-1, H, maps, dv) - want[rows]).abs().max()
+    assert float(err) < 3e-4, float(err)
+    got = mx.attention(qd, kc, vc, pos, seq, table, bs, H * maps, maps, H // G, d, dv, 0.2, mask, size, 1, False,
+                       tiles, n_pre)
+    assert float((got.cpu().double().view(-1, H, maps, dv) - want[rows]).abs().max()) < 3e-2
 
 
 @pytest.mark.parametrize("device", DEVICES)
