@@ -146,6 +146,9 @@ def parse(argv=None):
                          "prefilled with this probability -- blocks allocated, KV taken as arrived -- so one GPU "
                          "measures the decode role of an xPyD layout whose decode engines prefill the other "
                          "1 - q of the prompts locally (1 = pure decode role)")
+    ap.add_argument("--layered", action="store_true",
+                    help="instead of the headline workload: the layer-listed model family (Bekulix) beside Llama at "
+                         "equal layer sizes, prefill / decode tokens/s and attention kernels alone (one GPU)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--gemm-report", default=None, help="write the decode-GEMM tuning table (JSON) here")
     ap.add_argument("--seed", type=int, default=0)
@@ -422,6 +425,11 @@ def main(argv=None):
         torch.cuda.set_device(local)
         dev = torch.device("cuda", local)
     extra: dict = {}
+    if args.layered:
+        from dynamo_exp_amd.bench.layered import run_layered_compare
+
+        print(json.dumps(run_layered_compare(args, dev)), flush=True)
+        return
     if world > 1 and args.mode == "agg":
         from dynamo_exp_amd.bench.dp import run_data_parallel
 

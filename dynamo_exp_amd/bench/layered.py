@@ -1,0 +1,163 @@
+"""`bench.py --layered`: a layer-listed model (Bekulix) beside the closest
+existing model (Llama) at equal layer sizes, random weights.
+
+Two parts, both on one GPU:
+  * engine throughput through the engine's own entry point (add_request +
+    step: scheduler, paged caches, HIP graphs for decode, greedy sampling):
+    one prefill step of `prefill_seqs` x `isl` tokens, then decode of
+    `decode_seqs` streams at context `isl` for `osl` tokens;
+  * the attention kernels alone at the layer's head shape: matrix-core
+    prefill kernels in TFLOP/s (causal FLOPs 4 d L^2 / 2 per head), decode
+    kernels in TB/s of cache bytes read -- each kernel's distance from its
+    roofline, Bekulix's next to Llama's.
+"""
+from __future__ import annotations
+
+import math
+import time
+
+import torch
+
+from .. import ops
+from ..engine.engine import EngineConfig, LLMEngine
+from ..engine.request import SamplingParams
+from ..models.config import ModelConfig, _bekulix_preset
+from ..ops import mixers as mx
+
+# layer sizes of real models (width, ff, heads, kv heads, head dim), a few layers each
+SIZES = {
+    "1b-shapes": dict(W=2048, ff=8192, H=16, G=4, d=128, layers=8, vocab=32000),
+    "8b-shapes": dict(W=4096, ff=14336, H=32, G=8, d=128, layers=8, vocab=128256),
+}
+
+
+def _configs(s: dict):
+    bek = _bekulix_preset(f"bekulix {s['W']}", s["W"], s["ff"], s["layers"], s["H"], s["G"], s["d"], 256, 1024, 2048,
+                          vocab=s["vocab"])
+    lla = ModelConfig(name=f"llama {s['W']}", vocab_size=s["vocab"], hidden_size=s["W"], intermediate_size=s["ff"],
+                      num_hidden_layers=s["layers"], num_attention_heads=s["H"], num_key_value_heads=s["G"],
+                      head_dim=s["d"], max_position_embeddings=8192, bos_token_id=1, eos_token_id=[2])
+    return bek, lla
+
+
+def _timed(fn, iters=10, warm=2) -> float:
+    for _ in range(warm):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) / iters * 1e3  # us
+
+
+def engine_throughput(mcfg, dev, isl: int, osl: int, prefill_seqs: int, decode_seqs: int, seed: int = 0) -> dict:
+    """Prefill and decode tokens/s of one model through LLMEngine."""
+    out = {}
+    g = torch.Generator().manual_seed(seed)
+    for phase, B in (("prefill", prefill_seqs), ("decode", decode_seqs)):
+        eng = LLMEngine(EngineConfig(model=mcfg.name, device=str(dev), block_size=64, max_model_len=isl + osl + 64,
+                                     max_num_seqs=B, max_num_batched_tokens=max(8192, prefill_seqs * isl),
+                                     chunked_prefill=False, max_prefill_streak=1 << 30, enable_prefix_caching=False,
+                                     num_gpu_blocks=B * (-(-(isl + osl + 64) // 64)) + 8, graph_sizes=(B,),
+                                     async_schedule=False, seed=seed), model_cfg=mcfg)
+        eng.warmup()
+        best = None
+        for rep in range(3):  # first repetition warms the GEMM library at these sizes
+            first = {}
+            for i in range(B):
+                p = torch.randint(3, mcfg.vocab_size, (isl,), generator=g).tolist()
+                eng.add_request(f"{phase}{rep}_{i}", p, SamplingParams(max_tokens=osl if phase == "decode" else 1,
+                                                                        ignore_eos=True),
+                                on_output=lambda r, t, lp, fin: first.setdefault(r.request_id, True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while len(first) < B:
+                eng.step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            while eng.has_unfinished():
+                eng.step()
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            v = B * isl / (t1 - t0) if phase == "prefill" else B * (osl - 1) / (t2 - t1)
+            if rep:
+                best = max(best or 0.0, v)
+        out[f"{phase}_tok_s"] = round(best, 1)
+        del eng
+        torch.cuda.empty_cache()
+    return out
+
+
+def attention_kernels(s: dict, L: int, B: int) -> dict:
+    """The attention kernels alone at head shape (H, G, d): one prompt of L
+    tokens (prefill) and B streams at context L (decode)."""
+    H, G, d, bs = s["H"], s["G"], s["d"], 64
+    dev, dt = "cuda", torch.bfloat16
+    res = {}
+    flops = 4 * d * H * L * (L + 1) / 2
+    nb = L // bs + 1
+    # ---- prefill
+    q = torch.randn(L, H * d, device=dev, dtype=dt)
+    pos = torch.arange(L, device=dev)
+    seq = torch.zeros(L, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
+    kc = torch.randn(nb * bs, G * d, device=dev, dtype=dt)
+    vc = torch.randn_like(kc)
+    tiles = torch.tensor(mx.tile_list(0, L), dtype=torch.int32, device=dev)
+    us = _timed(lambda: mx.attention(q, kc, vc, pos, seq, bt, bs, H, 1, H // G, d, d, d ** -0.5, "causal", 0, 1, False,
+                                     tiles, L))
+    res["bekulix_prefill_causal"] = {"us": round(us, 1), "TFLOPs": round(flops / us / 1e6, 1)}
+    for mask, size in (("window", 1024), ("chunk", 2048)):
+        j = torch.arange(L)
+        lo = mx.first_visible(j, mask, size)
+        fl = 4 * d * H * float((j - lo + 1).sum())
+        us = _timed(lambda: mx.attention(q, kc, vc, pos, seq, bt, bs, H, 1, H // G, d, d, d ** -0.5, mask, size, 1,
+                                         False, tiles, L))
+        res[f"bekulix_prefill_{mask}{size}"] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1)}
+    kl = torch.randn(nb, G, bs, d, device=dev, dtype=dt)
+    vl = torch.randn_like(kl)
+    ql = q.view(L, H, d)
+    cu = torch.tensor([0, L], dtype=torch.int32, device=dev)
+    ctx = torch.tensor([L], dtype=torch.int32, device=dev)
+    work = torch.tensor(ops.prefill_work_list([L], [L], H, G), dtype=torch.int32, device=dev)
+    out = torch.empty_like(ql)
+    us = _timed(lambda: ops.prefill_attention(ql, kl, vl, bt, cu, ctx, d ** -0.5, out, work=work))
+    res["llama_prefill_causal"] = {"us": round(us, 1), "TFLOPs": round(flops / us / 1e6, 1)}
+    # ---- decode
+    nbb = B * nb
+    byts = B * L * G * d * 2 * 2
+    bt = torch.randperm(nbb, device=dev).to(torch.int32).view(B, nb)
+    kc = torch.randn(nbb * bs, G * d, device=dev, dtype=dt)
+    vc = torch.randn_like(kc)
+    q = torch.randn(B, H * d, device=dev, dtype=dt)
+    pos = torch.full((B,), L - 1, device=dev)
+    parts = mx.row_attention_parts(B, G, L)
+    us = _timed(lambda: mx.attention(q, kc, vc, pos, None, bt, bs, H, 1, H // G, d, d, d ** -0.5, "causal", 0, parts))
+    res["bekulix_decode"] = {"us": round(us, 1), "TB/s": round(byts / us / 1e6, 2), "parts": parts}
+    kl = torch.randn(nbb, G, bs, d, device=dev, dtype=dt)
+    vl = torch.randn_like(kl)
+    ql = q.view(B, H, d)
+    ctx = torch.full((B,), L, dtype=torch.int32, device=dev)
+    out = torch.empty_like(ql)
+    mp = ops.decode_num_parts(B, G, L)
+    ws = ops.decode_workspace(B, H, d, mp, dev)
+    us = _timed(lambda: ops.decode_attention(ql, kl, vl, bt, ctx, d ** -0.5, out, mp, workspace=ws))
+    res["llama_decode"] = {"us": round(us, 1), "TB/s": round(byts / us / 1e6, 2), "parts": mp}
+    return res
+
+
+def run_layered_compare(args, dev) -> dict:
+    isl, osl = min(args.isl, 2048), min(args.osl, 64)
+    sizes = {}
+    for name, s in SIZES.items():
+        bek, lla = _configs(s)
+        row = {"layers": s["layers"], "isl": isl, "osl": osl, "prefill_seqs": 4, "decode_seqs": 64}
+        row["bekulix"] = engine_throughput(bek, dev, isl, osl, 4, 64, args.seed)
+        row["llama"] = engine_throughput(lla, dev, isl, osl, 4, 64, args.seed)
+        row["attention_kernels"] = attention_kernels(s, 4096, 64)
+        sizes[name] = row
+    return {"metric": "layer-listed model (Bekulix) beside Llama at equal layer sizes: engine prefill / decode "
+                      "tokens/s and attention kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic (random-token prompts, random-init weights)", "sizes": sizes}

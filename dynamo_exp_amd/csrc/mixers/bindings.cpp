@@ -27,6 +27,9 @@ int dxm_row_attention(void*, float*, const void*, int64_t, const void*, const vo
 int dxm_tile_attention_ok(int, int);
 int dxm_tile_attention(void*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*,
                        int, int, const int*, int, int, int, int, int, int, int, int, float, int, int, int, hipStream_t);
+int dxm_group_decode(float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*, int,
+                     int, int, int, int, int, int, int, int, int, float, int, int, int, hipStream_t);
+int dxm_merge_parts(void*, const float*, int64_t, int, int, int, hipStream_t);
 }
 
 static void check(int rc, const char* what) {
@@ -72,6 +75,15 @@ PYBIND11_MODULE(_C_mixers, m) {
                              reinterpret_cast<const int*>(tiles), n_tiles, n_qh, maps, group, d, dv, Wk, Wv, scale,
                              mask, size, out_f32, S(st)),
           "tile_attention");
+  });
+  m.def("group_decode", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
+                           int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
+                           int size, int parts, int out_f32, u st) {
+    check(dxm_group_decode(F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
+                           reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
+                           maps, group, d, dv, Wk, Wv, scale, mask, size, parts, S(st)),
+          "group_decode");
+    check(dxm_merge_parts(P(out), F(ws), (int64_t)rows * n_qh, parts, dv, out_f32, S(st)), "merge_parts");
   });
   m.def("row_attention", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                             int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,

@@ -222,3 +222,14 @@ extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_
   if (out_f32) return launch_rows<bf16_t, float>(a, rows, st);
   return launch_rows<bf16_t, bf16_t>(a, rows, st);
 }
+
+// out [n_vec, dv] (bf16 or fp32) from per-part partials ws [n_vec, parts, 2 + dv]
+extern "C" int dxm_merge_parts(void* out, const float* ws, int64_t n_vec, int parts, int dv, int out_f32,
+                               hipStream_t st) {
+  if (n_vec <= 0) return 0;
+  if (parts < 1 || dv < 1 || n_vec > 0x7fffffff) return 1;
+  if (out_f32) hipLaunchKernelGGL((merge_parts_kernel<float>), dim3((unsigned)n_vec), dim3(64), 0, st, (float*)out, ws, parts, dv);
+  else hipLaunchKernelGGL((merge_parts_kernel<bf16_t>), dim3((unsigned)n_vec), dim3(64), 0, st, (bf16_t*)out, ws, parts, dv);
+  DX_CHECK_LAUNCH();
+  return 0;
+}

@@ -49,6 +49,36 @@ __device__ __forceinline__ int64_t first_visible(int64_t p, int mask, int size) 
   return 0;
 }
 
+// Stage keys kt .. kt + 63 (those <= hi; the rest as zeros) of one K head and one
+// V head into LDS: K row-major [64][d + 8], V transposed [dv][64 + 8].  NT
+// threads, 4 per key and pass.
+template <int d, int dv, int NT>
+__device__ __forceinline__ void stage_tile(bf16_t* Ks, bf16_t* Vt, const bf16_t* kc, const bf16_t* vc, const int* bt,
+                                           int bs, int Wk, int Wv, int64_t kt, int64_t hi, int tid) {
+  constexpr int ks_stride = d + 8;
+#pragma unroll
+  for (int base = 0; base < 256; base += NT) {
+    const int t = base + tid;
+    const int key = t >> 2, part = t & 3;
+    const int64_t kj = kt + key;
+    const bool ok = kj <= hi;
+    const int64_t slot = ok ? (int64_t)bt[kj / bs] * bs + kj % bs : 0;
+    const bf16_t* ksrc = kc + slot * Wk;
+    const bf16_t* vsrc = vc + slot * Wv;
+    const u16x8 zero = {{0, 0, 0, 0}};
+    for (int c = part * 8; c < d; c += 32)
+      *reinterpret_cast<u16x8*>(Ks + key * ks_stride + c) = ok ? *reinterpret_cast<const u16x8*>(ksrc + c) : zero;
+    for (int c = part * 8; c < dv; c += 32) {
+      const u16x8 v = ok ? *reinterpret_cast<const u16x8*>(vsrc + c) : zero;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        Vt[(c + 2 * i) * kVtStride + key] = (bf16_t)(v.w[i] & 0xffffu);
+        Vt[(c + 2 * i + 1) * kVtStride + key] = (bf16_t)(v.w[i] >> 16);
+      }
+    }
+  }
+}
+
 template <typename OutT> __device__ __forceinline__ void store4(OutT* o, f32x4 v);
 template <> __device__ __forceinline__ void store4<float>(float* o, f32x4 v) { *reinterpret_cast<f32x4*>(o) = v; }
 template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* o, f32x4 v) {
@@ -100,25 +130,7 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   for (int64_t kt = kt0; kt <= hi; kt += kKeys) {
-    {  // stage the tile: 4 threads per key
-      const int key = tid >> 2, part = tid & 3;
-      const int64_t kj = kt + key;
-      const bool ok = kj <= hi;
-      const int64_t slot = ok ? (int64_t)bt[kj / a.bs] * a.bs + kj % a.bs : 0;
-      const bf16_t* ksrc = kc + slot * a.Wk;
-      const bf16_t* vsrc = vc + slot * a.Wv;
-      const u16x8 zero = {{0, 0, 0, 0}};
-      for (int c = part * 8; c < d; c += 32)
-        *reinterpret_cast<u16x8*>(Ks + key * ks_stride + c) = ok ? *reinterpret_cast<const u16x8*>(ksrc + c) : zero;
-      for (int c = part * 8; c < dv; c += 32) {
-        const u16x8 v = ok ? *reinterpret_cast<const u16x8*>(vsrc + c) : zero;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          Vt[(c + 2 * i) * kVtStride + key] = (bf16_t)(v.w[i] & 0xffffu);
-          Vt[(c + 2 * i + 1) * kVtStride + key] = (bf16_t)(v.w[i] >> 16);
-        }
-      }
-    }
+    stage_tile<d, dv, 256>(Ks, Vt, kc, vc, bt, a.bs, a.Wk, a.Wv, kt, hi, tid);
     __syncthreads();
     if (wave_on) {
       f32x4 S[2][4];
@@ -199,6 +211,181 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// Decode rows: one wave per (row, K head, chunk of the heads that share it,
+// key part).  The 16 B-operand columns are query heads of one group instead of
+// 16 consecutive tokens, so the K/V bytes of a group are read once for all its
+// heads; everything else is the tile kernel's arithmetic.  The wave's partial
+// (max, sum, acc) go to the workspace that merge_parts (row_attention.hip)
+// joins: ws [rows, n_qh, parts, 2 + dv].
+struct GroupArgs {
+  const bf16_t* q;
+  int64_t q_stride;
+  const bf16_t* kc;
+  const bf16_t* vc;
+  float* ws;
+  const int64_t* pos;
+  const int* seq;  // null: row i is sequence i
+  const int* bt;
+  int bt_stride, bs;
+  int n_qh, maps, group, chunks;
+  int Wk, Wv;
+  float scale;
+  int mask, size, parts;
+};
+
+template <int DB, int DVB, int QB>
+__global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
+  constexpr int d = DB * 16, dv = DVB * 16, ks_stride = d + 8;
+  extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+  bf16_t* Ks = smem;
+  bf16_t* Vt = smem + kKeys * ks_stride;
+  const int lane = threadIdx.x, c16 = lane & 15, g4 = lane >> 4;
+  const int gm = blockIdx.x / a.chunks, chunk = blockIdx.x - gm * a.chunks;
+  const int g = gm / a.maps, m = gm - g * a.maps;
+  const int row = blockIdx.y, part = blockIdx.z;
+  const int64_t p = a.pos[row];
+  const int* bt = a.bt + (int64_t)(a.seq ? a.seq[row] : row) * a.bt_stride;
+  const bf16_t* kc = a.kc + (int64_t)gm * d;
+  const bf16_t* vc = a.vc + (int64_t)g * dv;
+  const int64_t lo = first_visible(p, a.mask, a.size);
+  const int64_t tiles = (p - lo + kKeys) / kKeys;
+  const int64_t tpp = (tiles + a.parts - 1) / a.parts;
+  const int64_t t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
+
+  i16x4 qf[QB][DB];
+  bool okh[QB];
+  int qh[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int hi_ = chunk * 16 * QB + 16 * qb + c16;
+    okh[qb] = hi_ < a.group;
+    qh[qb] = (g * a.group + (okh[qb] ? hi_ : 0)) * a.maps + m;
+    const bf16_t* q = a.q + (int64_t)row * a.q_stride + (int64_t)qh[qb] * d + 4 * g4;
+#pragma unroll
+    for (int ks = 0; ks < DB; ++ks)
+      qf[qb][ks] = okh[qb] ? *reinterpret_cast<const i16x4*>(q + ks * 16) : i16x4{0, 0, 0, 0};
+  }
+  float mx[QB], lsum[QB];
+  f32x4 O[QB][DVB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    mx[qb] = -INFINITY;
+    lsum[qb] = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int64_t t = t0; t < t1; ++t) {
+    const int64_t kt = lo + t * kKeys;
+    stage_tile<d, dv, 64>(Ks, Vt, kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+    __syncthreads();
+    f32x4 S[QB][4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) S[qb][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DB; ++ks) {
+        const i16x4 A = *reinterpret_cast<const i16x4*>(Ks + (kb * 16 + c16) * ks_stride + ks * 16 + 4 * g4);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb)
+          S[qb][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[qb][ks], S[qb][kb], 0, 0, 0);
+      }
+    }
+    i16x4 Ph[QB][4], Pl[QB][4];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int64_t kj = kt + kb * 16 + 4 * g4 + i;
+          const float s = kj <= p ? S[qb][kb][i] * a.scale : -INFINITY;
+          S[qb][kb][i] = s;
+          mloc = fmaxf(mloc, s);
+        }
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+      const float mn = fmaxf(mx[qb], mloc);  // finite: every visited tile holds a visible key
+      const float alpha = __expf(mx[qb] - mn);
+      mx[qb] = mn;
+      float add = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        float pw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pw[i] = __expf(S[qb][kb][i] - mn);
+          add += pw[i];
+        }
+        const uint32_t h01 = pack_bf16x2(pw[0], pw[1]), h23 = pack_bf16x2(pw[2], pw[3]);
+        const uint32_t l01 = pack_bf16x2(pw[0] - bf16lo(h01), pw[1] - bf16hi(h01));
+        const uint32_t l23 = pack_bf16x2(pw[2] - bf16lo(h23), pw[3] - bf16hi(h23));
+        Ph[qb][kb] = __builtin_bit_cast(i16x4, uint2{h01, h23});
+        Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
+      }
+      lsum[qb] = lsum[qb] * alpha + add;
+#pragma unroll
+      for (int cb = 0; cb < DVB; ++cb) O[qb][cb] *= alpha;
+    }
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int cb = 0; cb < DVB; ++cb) {
+        const i16x4 A = *reinterpret_cast<const i16x4*>(Vt + (cb * 16 + c16) * kVtStride + kb * 16 + 4 * g4);
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Ph[qb][kb], O[qb][cb], 0, 0, 0);
+          O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Pl[qb][kb], O[qb][cb], 0, 0, 0);
+        }
+      }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    float l = lsum[qb];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!okh[qb]) continue;
+    float* w = a.ws + (((int64_t)row * a.n_qh + qh[qb]) * a.parts + part) * (2 + dv);
+    if (g4 == 0) {
+      w[0] = mx[qb];
+      w[1] = l;
+    }
+#pragma unroll
+    for (int cb = 0; cb < DVB; ++cb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[2 + cb * 16 + 4 * g4 + i] = O[qb][cb][i];
+  }
+}
+
+template <int DB, int DVB>
+int launch_group(const GroupArgs& a0, int rows, hipStream_t st) {
+  const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * kVtStride) * sizeof(bf16_t);
+  GroupArgs a = a0;
+  const bool two = a.group > 16;
+  a.chunks = two ? (a.group + 31) / 32 : 1;
+  auto k1 = group_decode_kernel<DB, DVB, 1>;
+  auto k2 = group_decode_kernel<DB, DVB, 2>;
+  if (lds > 48 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      if (hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess ||
+          hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return 7;
+      raised = true;
+    }
+  }
+  const int n_gm = a.n_qh / a.group;  // K heads (kv heads x maps)
+  const dim3 grid(n_gm * a.chunks, rows, a.parts);
+  if (two) hipLaunchKernelGGL(k2, grid, dim3(64), lds, st, a);
+  else hipLaunchKernelGGL(k1, grid, dim3(64), lds, st, a);
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
 template <int DB, int DVB, typename OutT>
 int launch_tiles(const TileArgs& a, int n_tiles, hipStream_t st) {
   const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * kVtStride) * sizeof(bf16_t);
@@ -255,6 +442,31 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
   TILE_CASE(8, 8)
   TILE_CASE(8, 16)
   TILE_CASE(16, 16)
+  return 2;
+}
+
+#define GROUP_CASE(DB_, DVB_) \
+  if (d == DB_ * 16 && dv == DVB_ * 16) return launch_group<DB_, DVB_>(a, rows, st);
+
+// Decode rows (one token per row) on the matrix cores: partials into ws
+// [rows, n_qh, parts, 2 + dv]; dxm_merge_parts joins them.
+int dxm_group_decode(float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
+                     const int* seq, const int* bt, int bt_stride, int bs, int rows, int n_qh, int maps, int group,
+                     int d, int dv, int Wk, int Wv, float scale, int mask, int size, int parts, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || rows > 65535) return 1;
+  if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535) return 3;
+  if (!ws || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
+  GroupArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, ws, pos, seq, bt, bt_stride, bs,
+              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts};
+  GROUP_CASE(2, 2)
+  GROUP_CASE(3, 3)
+  GROUP_CASE(3, 6)
+  GROUP_CASE(4, 4)
+  GROUP_CASE(4, 8)
+  GROUP_CASE(8, 8)
+  GROUP_CASE(8, 16)
+  GROUP_CASE(16, 16)
   return 2;
 }
 

@@ -264,11 +264,15 @@ class BekulixForCausalLM:
         return self
 
     # ------------------------------------------------------------------ forward
-    def _parts(self, rows: int, n_qh: int, mask: str, size: int, meta: AttnMeta) -> int:
+    def _parts(self, rows: int, n_qh: int, mask: str, size: int, meta: AttnMeta, group: int = 1) -> int:
+        """Key partitions of the step's decode rows (rows that are no prompt-chunk tiles)."""
         vis = meta.max_ctx if meta.max_ctx else self.cfg.max_position_embeddings
         if mask != "causal":
             vis = min(vis, size)
-        return mx.row_attention_parts(rows, n_qh, vis)
+        if meta.is_prefill:
+            rows -= meta.num_prefill_tokens if self.dtype == torch.bfloat16 and self.device.type == "cuda" else 0
+        units = n_qh if self.dtype != torch.bfloat16 else max(1, n_qh // group) * (-(-group // 32))
+        return mx.row_attention_parts(max(rows, 1), units, vis)
 
     def _mix(self, L: dict, h: torch.Tensor, meta: AttnMeta, kc, vc, seq, tables, bs: int) -> torch.Tensor:
         m, T = L["m"], h.shape[0]
@@ -283,7 +287,7 @@ class BekulixForCausalLM:
             mx.headprep_cache(p, pos, slots, H, G, d, H * d, L["qn"], L["kn"], eps,
                               (qt["coef"], qt["every"]) if qt else None, kc, vc, v_mode=1)
             a = mx.attention(p, kc, vc, pos, seq, tables, bs, H, 1, H // G, d, d, m["scale"], "causal", 0,
-                             self._parts(T, H, "causal", 0, meta), False, *tl)
+                             self._parts(T, H, "causal", 0, meta, H // G), False, *tl)
             return torch.matmul(a.view(T, H * d), L["w_o"].t())
         if L["type"] == "latent_attention":
             r, dv, size = m["kv_rank"], m["vdim"], m["mask"]["size"]
@@ -292,7 +296,7 @@ class BekulixForCausalLM:
             # fold W_uk into the query: the latent cache is the one key/value head of every query head
             ql = torch.bmm(p[:, : H * d].view(T, H, d).transpose(0, 1), L["uk"]).transpose(0, 1).contiguous()
             a = mx.attention(ql.view(T, H * r), kc, kc, pos, seq, tables, bs, H, 1, H, r, r, m["scale"], "window",
-                             size, self._parts(T, H, "window", size, meta), False, *tl)
+                             size, self._parts(T, H, "window", size, meta, H), False, *tl)
             o = torch.bmm(a.transpose(0, 1), L["uv"]).transpose(0, 1).reshape(T, H * dv)
             return torch.matmul(o, L["w_o"].t())
         G, dv, size = m["kv_heads"], m["vdim"], m["mask"]["size"]
@@ -301,7 +305,7 @@ class BekulixForCausalLM:
         mx.headprep_cache(p, pos, slots, 0, 2 * G, d, qw, None, None, eps, None, kc, vc, v_mode=2, v_off=qw + kw,
                           v_w=G * dv)
         a = mx.attention(p, kc, vc, pos, seq, tables, bs, 2 * H, 2, H // G, d, dv, m["scale"], "chunk", size,
-                         self._parts(T, 2 * H, "chunk", size, meta), True, *tl)
+                         self._parts(T, 2 * H, "chunk", size, meta, H // G), True, *tl)
         o = mx.diff_combine(a.view(T, H, 2, dv), L["lam"], 1.0 - float(m["diff"]), eps, self.dtype)
         return torch.matmul(o, L["w_o"].t())
 

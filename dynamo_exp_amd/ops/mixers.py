@@ -181,7 +181,9 @@ def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor
 
 # ----------------------------------------------------------------- attention
 def row_attention_parts(rows: int, n_qh: int, max_visible: int) -> int:
-    """Key partitions per row so a launch has about ROW_TARGET_WAVES waves."""
+    """Key partitions per row so a launch has about ROW_TARGET_WAVES waves
+    (n_qh: the independent units per row -- query heads for the row kernel, K
+    heads for the grouped decode kernel)."""
     if rows <= 0:
         return 1
     want = -(-ROW_TARGET_WAVES // (rows * n_qh))
@@ -220,25 +222,38 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     does not apply) on the row kernel.  Same arguments and result as
     row_attention."""
     T = q.shape[0]
-    if tiles is None or n_tile_rows == 0 or not tile_attention_ok(q, d, dv):
+    if not tile_attention_ok(q, d, dv):
         return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
                              mask, size, parts, out_f32)
+    if tiles is None:
+        n_tile_rows = 0
     if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous() or \
-            q.stride(1) != 1 or seq is None or seq.dtype != torch.int32 or positions.dtype != torch.int64 or \
-            block_tables.dtype != torch.int32 or tiles.dtype != torch.int32 or not tiles.is_contiguous():
+            q.stride(1) != 1 or (seq is not None and seq.dtype != torch.int32) or positions.dtype != torch.int64 or \
+            block_tables.dtype != torch.int32 or block_tables.stride(1) != 1:
         raise TypeError("attention: bf16 caches, int32 seq / block_tables / tiles, int64 positions")
     if n_qh % maps or (n_qh // maps) % group or mask not in MASKS or (mask != "causal" and size < 1):
         raise ValueError("attention: bad head counts or mask")
+    if q.shape[1] < n_qh * d or kc.shape[-1] < n_qh // group * d or vc.shape[-1] < n_qh // maps // group * dv:
+        raise ValueError("attention: widths do not cover the heads")
+    if seq is None and block_tables.shape[0] < T:
+        raise ValueError("attention: fewer block-table rows than rows")
     odt = torch.float32 if out_f32 else q.dtype
     out = torch.empty((T, n_qh, dv), dtype=odt, device=q.device)
-    _m().tile_attention(out.data_ptr(), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), positions.data_ptr(),
-                        seq.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), block_size, tiles.data_ptr(),
-                        tiles.shape[0], n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale),
-                        MASKS[mask], int(size), int(out_f32), _stream())
-    if n_tile_rows < T:
-        r = slice(n_tile_rows, T)
-        out[r] = row_attention(q[r], kc, vc, positions[r], seq[r], block_tables, block_size, n_qh, maps, group, d, dv,
-                               scale, mask, size, parts, out_f32)
+    common = (block_tables.data_ptr(), block_tables.stride(0), block_size)
+    heads = (n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale), MASKS[mask], int(size))
+    if n_tile_rows:
+        if seq is None or tiles.dtype != torch.int32 or not tiles.is_contiguous():
+            raise TypeError("attention: prompt-chunk rows need seq and int32 tiles")
+        _m().tile_attention(out.data_ptr(), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
+                            positions.data_ptr(), seq.data_ptr(), *common, tiles.data_ptr(), tiles.shape[0], *heads,
+                            int(out_f32), _stream())
+    n_dec = T - n_tile_rows
+    if n_dec:  # decode rows: the heads of a K/V group share one wave's key tiles
+        r0 = n_tile_rows
+        ws = torch.empty((n_dec, n_qh, parts, 2 + dv), dtype=torch.float32, device=q.device)
+        _m().group_decode(out[r0:].data_ptr(), ws.data_ptr(), q[r0:].data_ptr(), q.stride(0), kc.data_ptr(),
+                          vc.data_ptr(), positions[r0:].data_ptr(), _ptr(seq[r0:] if seq is not None else None),
+                          *common, n_dec, *heads, parts, int(out_f32), _stream())
     return out
 
 

@@ -196,7 +196,8 @@ def test_row_attention_alone(device, mask, size, dims):
 @pytest.mark.gpu
 @pytest.mark.parametrize("mask,size", [("causal", 0), ("window", 70), ("window", 3), ("chunk", 50), ("chunk", 200)])
 @pytest.mark.parametrize("dims", [(4, 2, 1, 32, 32), (2, 1, 2, 64, 128), (3, 3, 1, 128, 128), (2, 2, 1, 48, 48),
-                                  (2, 1, 1, 256, 256), (2, 1, 2, 128, 256), (2, 2, 2, 48, 96)])
+                                  (2, 1, 1, 256, 256), (2, 1, 2, 128, 256), (2, 2, 2, 48, 96), (40, 1, 1, 64, 64),
+                                  (20, 1, 1, 32, 32)])
 def test_tile_attention_alone(mask, size, dims):
     """The matrix-core prefill kernel: a 263-row portion that starts at position
     37 of a cached prefix (three tiles, the last ragged, cut inside pages,
@@ -232,9 +233,14 @@ def test_tile_attention_alone(mask, size, dims):
                        n_pre)
     err = (got.cpu().double().view(-1, H, maps, dv) - want[rows]).abs().max()
     assert float(err) < 3e-4, float(err)
-    got = mx.attention(qd, kc, vc, pos, seq, table, bs, H * maps, maps, H // G, d, dv, 0.2, mask, size, 1, False,
+    got = mx.attention(qd, kc, vc, pos, seq, table, bs, H * maps, maps, H // G, d, dv, 0.2, mask, size, 3, False,
                        tiles, n_pre)
     assert float((got.cpu().double().view(-1, H, maps, dv) - want[rows]).abs().max()) < 3e-2
+    # decode rows alone (row i = sequence i), keys split into parts
+    dr = torch.tensor([0, 1, 63, 64, 65, 255, 299], device="cuda")
+    got = mx.attention(q.reshape(T, -1).cuda()[dr], kc, vc, dr, None, table[:1].expand(len(dr), -1).contiguous(), bs,
+                       H * maps, maps, H // G, d, dv, 0.2, mask, size, 2, True)
+    assert float((got.cpu().double().view(-1, H, maps, dv) - want[dr.cpu()]).abs().max()) < 3e-4
 
 
 @pytest.mark.parametrize("device", DEVICES)
