@@ -43,41 +43,92 @@ struct TileArgs {
   int mask, size;
 };
 
-__device__ __forceinline__ int64_t first_visible(int64_t p, int mask, int size) {
+// positions are < 2^31: 32-bit arithmetic in the kernels
+__device__ __forceinline__ int first_visible(int p, int mask, int size) {
   if (mask == 1) return p - size + 1 > 0 ? p - size + 1 : 0;
-  if (mask == 2) return p / size * size;
+  if (mask == 2) return (int)((unsigned)p / (unsigned)size) * size;
   return 0;
 }
 
-// Stage keys kt .. kt + 63 (those <= hi; the rest as zeros) of one K head and one
-// V head into LDS: K row-major [64][d + 8], V transposed [dv][64 + 8].  NT
-// threads, 4 per key and pass.
+// A 64-key tile of one K head and one V head on its way from the paged caches
+// to LDS, split in two so the next tile's global loads fly during the current
+// tile's MFMAs: fetch() global -> registers, commit() registers -> LDS (K
+// row-major [64][d + 8]; V transposed [dv][64 + 8], four keys of one column
+// per 8-byte store).  Keys beyond `hi` arrive as zeros.  NT threads; work items
+// are 16-byte chunks, consecutive threads on consecutive chunks of a row.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 template <int d, int dv, int NT>
-__device__ __forceinline__ void stage_tile(bf16_t* Ks, bf16_t* Vt, const bf16_t* kc, const bf16_t* vc, const int* bt,
-                                           int bs, int Wk, int Wv, int64_t kt, int64_t hi, int tid) {
-  constexpr int ks_stride = d + 8;
+struct TileStage {
+  static constexpr int ks_stride = d + 8;
+  static constexpr int kItems = kKeys * (d / 8), vItems = (kKeys / 4) * (dv / 8);
+  static constexpr int kPer = (kItems + NT - 1) / NT, vPer = (vItems + NT - 1) / NT;
+  u32x4 kr[kPer];
+  u32x4 vr[vPer][4];
+
+  // slot of sequence position kj: block-table lookup in 32-bit arithmetic (a shift
+  // for the usual power-of-two block sizes; 64-bit divisions here cost more than the loads)
+  static __device__ __forceinline__ int64_t slot_of(const int* bt, int bs, int kj) {
+    const unsigned u = (unsigned)kj, b = (unsigned)bs;
+    if ((b & (b - 1)) == 0) {
+      const int sh = __builtin_ctz(b);
+      return ((int64_t)bt[u >> sh] << sh) + (u & (b - 1));
+    }
+    return (int64_t)bt[u / b] * bs + u % b;
+  }
+
+  __device__ __forceinline__ void fetch(const bf16_t* kc, const bf16_t* vc, const int* bt, int bs, int Wk, int Wv,
+                                        int kt, int hi, int tid) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    // One block-table lookup per lane (key kt + lane), handed to the lanes that load
+    // the key by a cross-lane read: a lookup per 16-byte load would put a dependent
+    // global round trip in front of each of them, and the loads retire in order.
+    const int mine = kt + (tid & 63) <= hi ? (int)slot_of(bt, bs, kt + (tid & 63)) : -1;
 #pragma unroll
-  for (int base = 0; base < 256; base += NT) {
-    const int t = base + tid;
-    const int key = t >> 2, part = t & 3;
-    const int64_t kj = kt + key;
-    const bool ok = kj <= hi;
-    const int64_t slot = ok ? (int64_t)bt[kj / bs] * bs + kj % bs : 0;
-    const bf16_t* ksrc = kc + slot * Wk;
-    const bf16_t* vsrc = vc + slot * Wv;
-    const u16x8 zero = {{0, 0, 0, 0}};
-    for (int c = part * 8; c < d; c += 32)
-      *reinterpret_cast<u16x8*>(Ks + key * ks_stride + c) = ok ? *reinterpret_cast<const u16x8*>(ksrc + c) : zero;
-    for (int c = part * 8; c < dv; c += 32) {
-      const u16x8 v = ok ? *reinterpret_cast<const u16x8*>(vsrc + c) : zero;
+    for (int i = 0; i < kPer; ++i) {
+      const int it = tid + i * NT;
+      const int key = it / (d / 8), ch = it % (d / 8);
+      const int64_t slot = __shfl(mine, key & 63, 64);
+      const bool ok = it < kItems && slot >= 0;
+      kr[i] = ok ? *reinterpret_cast<const u32x4*>(kc + slot * Wk + ch * 8) : zero;
+    }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        Vt[(c + 2 * i) * kVtStride + key] = (bf16_t)(v.w[i] & 0xffffu);
-        Vt[(c + 2 * i + 1) * kVtStride + key] = (bf16_t)(v.w[i] >> 16);
+    for (int i = 0; i < vPer; ++i) {
+      const int it = tid + i * NT;
+      const int kg = it / (dv / 8), ch = it % (dv / 8);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int64_t slot = __shfl(mine, (4 * kg + k) & 63, 64);
+        const bool ok = it < vItems && slot >= 0;
+        vr[i][k] = ok ? *reinterpret_cast<const u32x4*>(vc + slot * Wv + ch * 8) : zero;
       }
     }
   }
-}
+
+  __device__ __forceinline__ void commit(bf16_t* Ks, bf16_t* Vt, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int it = tid + i * NT;
+      if (it < kItems) *reinterpret_cast<u32x4*>(Ks + (it / (d / 8)) * ks_stride + (it % (d / 8)) * 8) = kr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < vPer; ++i) {
+      const int it = tid + i * NT;
+      if (it >= vItems) continue;
+      const int kg = it / (dv / 8), ch = it % (dv / 8);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {  // columns ch * 8 + 2 w, + 1: the four keys' values side by side
+        uint2 lo, hi2;
+        lo.x = (vr[i][0][w] & 0xffffu) | (vr[i][1][w] << 16);
+        lo.y = (vr[i][2][w] & 0xffffu) | (vr[i][3][w] << 16);
+        hi2.x = (vr[i][0][w] >> 16) | (vr[i][1][w] & 0xffff0000u);
+        hi2.y = (vr[i][2][w] >> 16) | (vr[i][3][w] & 0xffff0000u);
+        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w) * kVtStride + 4 * kg) = lo;
+        *reinterpret_cast<uint2*>(Vt + (ch * 8 + 2 * w + 1) * kVtStride + 4 * kg) = hi2;
+      }
+    }
+  }
+};
 
 template <typename OutT> __device__ __forceinline__ void store4(OutT* o, f32x4 v);
 template <> __device__ __forceinline__ void store4<float>(float* o, f32x4 v) { *reinterpret_cast<f32x4*>(o) = v; }
@@ -98,17 +149,17 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
   const int c16 = lane & 15, g4 = lane >> 4;
   const int qh = blockIdx.x;
   const int row0 = a.tiles[2 * blockIdx.y], n = a.tiles[2 * blockIdx.y + 1];
-  const int64_t p0 = a.pos[row0];
+  const int p0 = (int)a.pos[row0];
   const int* bt = a.bt + (int64_t)a.seq[row0] * a.bt_stride;
   const int head = qh / a.maps, m = qh - head * a.maps, g = head / a.group;
   const bf16_t* kc = a.kc + (int64_t)(g * a.maps + m) * d;
   const bf16_t* vc = a.vc + (int64_t)g * dv;
-  const int64_t hi = p0 + n - 1;
-  const int64_t kt0 = first_visible(p0, a.mask, a.size) / kKeys * kKeys;
+  const int hi = p0 + n - 1;
+  const int kt0 = first_visible(p0, a.mask, a.size) / kKeys * kKeys;
 
   // this wave's query fragments and per-row constants
   i16x4 qf[2][DB];
-  int64_t prow[2], lrow[2];
+  int prow[2], lrow[2];
   bool okrow[2];
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
@@ -129,9 +180,12 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int64_t kt = kt0; kt <= hi; kt += kKeys) {
-    stage_tile<d, dv, 256>(Ks, Vt, kc, vc, bt, a.bs, a.Wk, a.Wv, kt, hi, tid);
+  TileStage<d, dv, 256> stage;
+  stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt0, hi, tid);
+  for (int kt = kt0; kt <= hi; kt += kKeys) {
+    stage.commit(Ks, Vt, tid);
     __syncthreads();
+    if (kt + kKeys <= hi) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, hi, tid);
     if (wave_on) {
       f32x4 S[2][4];
 #pragma unroll
@@ -152,7 +206,7 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int64_t kj = kt + kb * 16 + 4 * g4 + i;
+            const int kj = kt + kb * 16 + 4 * g4 + i;
             const bool vis = okrow[qb] && kj >= lrow[qb] && kj <= prow[qb];
             const float s = vis ? S[qb][kb][i] * a.scale : -INFINITY;
             S[qb][kb][i] = s;
@@ -245,14 +299,14 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   const int gm = blockIdx.x / a.chunks, chunk = blockIdx.x - gm * a.chunks;
   const int g = gm / a.maps, m = gm - g * a.maps;
   const int row = blockIdx.y, part = blockIdx.z;
-  const int64_t p = a.pos[row];
+  const int p = (int)a.pos[row];
   const int* bt = a.bt + (int64_t)(a.seq ? a.seq[row] : row) * a.bt_stride;
   const bf16_t* kc = a.kc + (int64_t)gm * d;
   const bf16_t* vc = a.vc + (int64_t)g * dv;
-  const int64_t lo = first_visible(p, a.mask, a.size);
-  const int64_t tiles = (p - lo + kKeys) / kKeys;
-  const int64_t tpp = (tiles + a.parts - 1) / a.parts;
-  const int64_t t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
+  const int lo = first_visible(p, a.mask, a.size);
+  const int tiles = (p - lo + kKeys) / kKeys;
+  const int tpp = (tiles + a.parts - 1) / a.parts;
+  const int t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
 
   i16x4 qf[QB][DB];
   bool okh[QB];
@@ -276,10 +330,13 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  for (int64_t t = t0; t < t1; ++t) {
-    const int64_t kt = lo + t * kKeys;
-    stage_tile<d, dv, 64>(Ks, Vt, kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+  TileStage<d, dv, 64> stage;
+  if (t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, lo + t0 * kKeys, p, lane);
+  for (int t = t0; t < t1; ++t) {
+    const int kt = lo + t * kKeys;
+    stage.commit(Ks, Vt, lane);
     __syncthreads();
+    if (t + 1 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, p, lane);
     f32x4 S[QB][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -301,7 +358,7 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int64_t kj = kt + kb * 16 + 4 * g4 + i;
+          const int kj = kt + kb * 16 + 4 * g4 + i;
           const float s = kj <= p ? S[qb][kb][i] * a.scale : -INFINITY;
           S[qb][kb][i] = s;
           mloc = fmaxf(mloc, s);
