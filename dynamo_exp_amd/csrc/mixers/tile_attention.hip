@@ -130,6 +130,14 @@ struct TileStage {
   }
 };
 
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+// two 4-element fragments side by side as one K = 32 MFMA operand: slots 0..3 and
+// 4..7 of a lane group may hold any 8 of the 32 reduction indices, as long as
+// A and B agree -- here the lane group's 4 keys of two neighbouring 16-key blocks
+__device__ __forceinline__ bf16x8_t pair8(i16x4 a, i16x4 b) {
+  return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
 template <typename OutT> __device__ __forceinline__ void store4(OutT* o, f32x4 v);
 template <> __device__ __forceinline__ void store4<float>(float* o, f32x4 v) { *reinterpret_cast<f32x4*>(o) = v; }
 template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* o, f32x4 v) {
@@ -140,15 +148,19 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* o, f32x4 v) {
 }
 
 template <int DB, int DVB, typename OutT>
-__global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
+__global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_kernel(TileArgs a) {
   constexpr int d = DB * 16, dv = DVB * 16, ks_stride = d + 8;
+  constexpr bool X32 = DB % 2 == 0;  // d a multiple of 32: the K = 32 MFMA for the scores too
+  constexpr int DB2 = X32 ? DB / 2 : 1;
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
   bf16_t* Ks = smem;                    // [64][d + 8]
   bf16_t* Vt = smem + kKeys * ks_stride;  // [dv][64 + 8]
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int c16 = lane & 15, g4 = lane >> 4;
   const int qh = blockIdx.x;
-  const int row0 = a.tiles[2 * blockIdx.y], n = a.tiles[2 * blockIdx.y + 1];
+  // later tiles of a prompt see more keys: hand them out first (longest first)
+  const int ti = gridDim.y - 1 - blockIdx.y;
+  const int row0 = a.tiles[2 * ti], n = a.tiles[2 * ti + 1];
   const int p0 = (int)a.pos[row0];
   const int* bt = a.bt + (int64_t)a.seq[row0] * a.bt_stride;
   const int head = qh / a.maps, m = qh - head * a.maps, g = head / a.group;
@@ -159,6 +171,7 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
 
   // this wave's query fragments and per-row constants
   i16x4 qf[2][DB];
+  bf16x8_t qf8[2][DB2];
   int prow[2], lrow[2];
   bool okrow[2];
 #pragma unroll
@@ -168,11 +181,19 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
     prow[qb] = p0 + r;
     lrow[qb] = first_visible(prow[qb], a.mask, a.size);
     const bf16_t* q = a.q + (int64_t)(row0 + (okrow[qb] ? r : 0)) * a.q_stride + (int64_t)qh * d + 4 * g4;
+    if constexpr (X32) {
 #pragma unroll
-    for (int ks = 0; ks < DB; ++ks)
-      qf[qb][ks] = okrow[qb] ? *reinterpret_cast<const i16x4*>(q + ks * 16) : i16x4{0, 0, 0, 0};
+      for (int ks = 0; ks < DB2; ++ks)
+        qf8[qb][ks] = okrow[qb] ? *reinterpret_cast<const bf16x8_t*>(q + 4 * g4 + ks * 32)
+                                : __builtin_bit_cast(bf16x8_t, i16x8{0, 0, 0, 0, 0, 0, 0, 0});
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < DB; ++ks)
+        qf[qb][ks] = okrow[qb] ? *reinterpret_cast<const i16x4*>(q + ks * 16) : i16x4{0, 0, 0, 0};
+    }
   }
   const bool wave_on = 32 * w < n;
+  const float sc2 = a.scale * 1.4426950408889634f;  // scores in log2 units: exp2 is one instruction
   float mx[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
   f32x4 O[2][DVB];
 #pragma unroll
@@ -191,13 +212,26 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
         S[0][kb] = S[1][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (X32) {
 #pragma unroll
-        for (int ks = 0; ks < DB; ++ks) {
-          const i16x4 A = *reinterpret_cast<const i16x4*>(Ks + (kb * 16 + c16) * ks_stride + ks * 16 + 4 * g4);
-          S[0][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[0][ks], S[0][kb], 0, 0, 0);
-          S[1][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[1][ks], S[1][kb], 0, 0, 0);
+          for (int ks = 0; ks < DB2; ++ks) {
+            const bf16x8_t A =
+                *reinterpret_cast<const bf16x8_t*>(Ks + (kb * 16 + c16) * ks_stride + ks * 32 + 8 * g4);
+            S[0][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, qf8[0][ks], S[0][kb], 0, 0, 0);
+            S[1][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, qf8[1][ks], S[1][kb], 0, 0, 0);
+          }
+        } else {
+#pragma unroll
+          for (int ks = 0; ks < DB; ++ks) {
+            const i16x4 A = *reinterpret_cast<const i16x4*>(Ks + (kb * 16 + c16) * ks_stride + ks * 16 + 4 * g4);
+            S[0][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[0][ks], S[0][kb], 0, 0, 0);
+            S[1][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[1][ks], S[1][kb], 0, 0, 0);
+          }
         }
       }
+      // a tile every row of the wave sees whole needs no per-element mask
+      const bool full = 32 * w + 31 < n && kt + kKeys - 1 <= p0 + 32 * w &&
+                        kt >= first_visible(p0 + 32 * w + 31, a.mask, a.size);
       i16x4 Ph[2][4], Pl[2][4];
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb) {
@@ -207,8 +241,8 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int kj = kt + kb * 16 + 4 * g4 + i;
-            const bool vis = okrow[qb] && kj >= lrow[qb] && kj <= prow[qb];
-            const float s = vis ? S[qb][kb][i] * a.scale : -INFINITY;
+            const bool vis = full || (okrow[qb] && kj >= lrow[qb] && kj <= prow[qb]);
+            const float s = vis ? S[qb][kb][i] * sc2 : -INFINITY;  // log2 units
             S[qb][kb][i] = s;
             mloc = fmaxf(mloc, s);
           }
@@ -216,7 +250,7 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
         const float mn = fmaxf(mx[qb], mloc);
         const float mu = mn == -INFINITY ? 0.f : mn;  // a row that sees nothing in this tile
-        const float alpha = __expf(mx[qb] - mu);
+        const float alpha = fast_exp2(mx[qb] - mu);
         mx[qb] = mn;
         float add = 0.f;
 #pragma unroll
@@ -224,7 +258,7 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
           float p[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            p[i] = __expf(S[qb][kb][i] - mu);
+            p[i] = fast_exp2(S[qb][kb][i] - mu);
             add += p[i];
           }
           const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
@@ -238,16 +272,24 @@ __global__ void __launch_bounds__(256) tile_attention_kernel(TileArgs a) {
         for (int cb = 0; cb < DVB; ++cb) O[qb][cb] *= alpha;
       }
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
+      for (int kp = 0; kp < 2; ++kp) {  // 32 keys per MFMA: key blocks 2 kp and 2 kp + 1
+        bf16x8_t Bh[2], Bl[2];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          Bh[qb] = pair8(Ph[qb][2 * kp], Ph[qb][2 * kp + 1]);
+          Bl[qb] = pair8(Pl[qb][2 * kp], Pl[qb][2 * kp + 1]);
+        }
 #pragma unroll
         for (int cb = 0; cb < DVB; ++cb) {
-          const i16x4 A = *reinterpret_cast<const i16x4*>(Vt + (cb * 16 + c16) * kVtStride + kb * 16 + 4 * g4);
+          const bf16_t* vrow = Vt + (cb * 16 + c16) * kVtStride + kp * 32 + 4 * g4;
+          const bf16x8_t A = pair8(*reinterpret_cast<const i16x4*>(vrow), *reinterpret_cast<const i16x4*>(vrow + 16));
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
-            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Ph[qb][kb], O[qb][cb], 0, 0, 0);
-            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, Pl[qb][kb], O[qb][cb], 0, 0, 0);
+            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, Bh[qb], O[qb][cb], 0, 0, 0);
+            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, Bl[qb], O[qb][cb], 0, 0, 0);
           }
         }
+      }
     }
     __syncthreads();
   }
@@ -488,7 +530,7 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
   if (n_tiles <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1)) return 3;
-  if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
+  if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 8) return 4;
   TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
              tiles, n_qh, maps, group, Wk, Wv, scale, mask, size};
   TILE_CASE(2, 2)
