@@ -55,6 +55,8 @@ def parse_args(argv: list[str]):
     ap = argparse.ArgumentParser(prog="run")
     ap.add_argument("--model-path", default=os.environ.get("DX_MODEL", "llama3-8b"))
     ap.add_argument("--model-name", default=None)
+    ap.add_argument("--dtype", default=None, choices=["bfloat16", "float32"],
+                    help="activation / weight dtype (float32: models with 32-bit kernels, models/registry.py)")
     ap.add_argument("--model-config", default=None)
     ap.add_argument("--http-port", type=int, default=8080)
     ap.add_argument("--http-host", default="0.0.0.0")
@@ -125,7 +127,7 @@ def make_native_engine(a):
     dev = f"cuda:{a.base_gpu_id}" if torch.cuda.is_available() else "cpu"
     cfg = EngineConfig.from_args(model=a.model_path, block_size=a.kv_cache_block_size, max_model_len=a.max_model_len,
                                  max_num_seqs=a.max_num_seqs, gpu_memory_utilization=a.gpu_memory_utilization,
-                                 use_cuda_graph=not a.no_graph, device=dev, **kw)
+                                 use_cuda_graph=not a.no_graph, device=dev, dtype=a.dtype, **kw)
     if a.tensor_parallel_size > 1:
         from ..parallel.tp import make_tp_engine
 

@@ -111,7 +111,11 @@ class LLMEngine:
         dev = torch.device(cfg.device)
         if model is None:
             model = build_model(self.model_cfg, device=dev, tp=tp, dtype=cfg.dtype)
-            if cfg.random_init or not os.path.isdir(cfg.model):
+            import glob
+
+            # a directory that holds weights is loaded; random weights of the architecture otherwise
+            has_weights = os.path.isdir(cfg.model) and bool(glob.glob(os.path.join(cfg.model, "*.safetensors")))
+            if not has_weights and (cfg.random_init or not os.path.isdir(cfg.model)):
                 model.random_init(cfg.seed)
             else:
                 model.load_safetensors(cfg.model)

@@ -48,6 +48,12 @@ from .llama import AttnMeta, TPGroup
 MIXER_TYPES = ("attention", "latent_attention", "attention_2")
 
 
+def _mask_of(m: dict, kind: str) -> tuple[str, int]:
+    """(mask kind, size) of a mixer whose mask is of `kind` when it gives a size, plain causal otherwise."""
+    size = (m.get("mask") or {}).get("size")
+    return (kind, int(size)) if size else ("causal", 0)
+
+
 class BekulixForCausalLM:
     #: the runner builds per-row sequence ids and one block table over all rows of a step
     unified_rows = True
@@ -290,22 +296,24 @@ class BekulixForCausalLM:
                              self._parts(T, H, "causal", 0, meta, H // G), False, *tl)
             return torch.matmul(a.view(T, H * d), L["w_o"].t())
         if L["type"] == "latent_attention":
-            r, dv, size = m["kv_rank"], m["vdim"], m["mask"]["size"]
+            r, dv = m["kv_rank"], m["vdim"]
+            mask, size = _mask_of(m, "window")
             p = torch.matmul(h, L["w_in"].t())
             mx.headprep_cache(p, pos, slots, 0, 1, r, H * d, None, L["cn"], eps, None, kc, None, v_mode=0)
             # fold W_uk into the query: the latent cache is the one key/value head of every query head
             ql = torch.bmm(p[:, : H * d].view(T, H, d).transpose(0, 1), L["uk"]).transpose(0, 1).contiguous()
-            a = mx.attention(ql.view(T, H * r), kc, kc, pos, seq, tables, bs, H, 1, H, r, r, m["scale"], "window",
-                             size, self._parts(T, H, "window", size, meta, H), False, *tl)
+            a = mx.attention(ql.view(T, H * r), kc, kc, pos, seq, tables, bs, H, 1, H, r, r, m["scale"], mask,
+                             size, self._parts(T, H, mask, size, meta, H), False, *tl)
             o = torch.bmm(a.transpose(0, 1), L["uv"]).transpose(0, 1).reshape(T, H * dv)
             return torch.matmul(o, L["w_o"].t())
-        G, dv, size = m["kv_heads"], m["vdim"], m["mask"]["size"]
+        G, dv = m["kv_heads"], m["vdim"]
+        mask, size = _mask_of(m, "chunk")
         p = torch.addmm(L["b_in"], h, L["w_in"].t())
         qw, kw = H * 2 * d, G * 2 * d
         mx.headprep_cache(p, pos, slots, 0, 2 * G, d, qw, None, None, eps, None, kc, vc, v_mode=2, v_off=qw + kw,
                           v_w=G * dv)
-        a = mx.attention(p, kc, vc, pos, seq, tables, bs, 2 * H, 2, H // G, d, dv, m["scale"], "chunk", size,
-                         self._parts(T, 2 * H, "chunk", size, meta, H // G), True, *tl)
+        a = mx.attention(p, kc, vc, pos, seq, tables, bs, 2 * H, 2, H // G, d, dv, m["scale"], mask, size,
+                         self._parts(T, 2 * H, mask, size, meta, H // G), True, *tl)
         o = mx.diff_combine(a.view(T, H, 2, dv), L["lam"], 1.0 - float(m["diff"]), eps, self.dtype)
         return torch.matmul(o, L["w_o"].t())
 

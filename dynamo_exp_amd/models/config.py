@@ -162,7 +162,7 @@ class LayeredConfig:
         if not lp:
             return list(range(n))
         a, b, times = int(lp["start"]), int(lp["stop"]), int(lp["times"])
-        if not (0 <= a <= b <= n and times >= 1):
+        if not (0 <= a <= b <= n and times >= 0):
             raise ValueError(f"bad loop {lp!r} for {n} layers")
         return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
