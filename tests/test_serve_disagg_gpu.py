@@ -185,6 +185,9 @@ def test_served_disagg_router_graph_one_gpu(tmp_path):
     _agg_then_disagg(tmp_path, "llama3-8b@8", "0.5", "host")
 
 
+@pytest.mark.skipif(os.environ.get("DX_RUN_XPROC_IPC") != "1",
+                    reason="cross-process dma-buf import of the KV cache hangs on these GPU boxes "
+                           "(DX_RUN_XPROC_IPC=1 to run; see tests/test_disagg_loopback.py)")
 @pytest.mark.gpu
 def test_served_disagg_router_graph_one_gpu_one_sided(tmp_path):
     """The same served graph with `--kv-transport ipc`: the prefill worker
