@@ -329,9 +329,8 @@ class LLMEngine:
         them whose logits are wanted), all in one batch through the scheduler's
         page management and the runner's forward.  Requests in `end` are
         finished afterwards.  Returns {request id: fp32 logits [n_wanted,
-        vocab]} for entries that wanted any."""
-        if self._cuda:
-            streams.enter_compute(self.model.device)
+        vocab]} for entries that wanted any.  Runs on the caller's current
+        stream (a replay samples nothing and needs none of the serving streams)."""
         if self._inflight is not None:
             raise RuntimeError("forced_step with a sampled batch in flight")
 
