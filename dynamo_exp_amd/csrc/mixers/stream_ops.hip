@@ -22,13 +22,38 @@ template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float
 template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
 
+// V consecutive elements as floats (V = 4: one 8-byte / 16-byte access; V = 1: scalar)
+template <typename T, int V> __device__ __forceinline__ void ldv(const T* p, float* o) {
+  if constexpr (V == 1) {
+    o[0] = ldf<T>(p, 0);
+  } else if constexpr (sizeof(T) == 2) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    o[0] = bf16lo(w.x), o[1] = bf16hi(w.x), o[2] = bf16lo(w.y), o[3] = bf16hi(w.y);
+  } else {
+    const f32x4 w = *reinterpret_cast<const f32x4*>(p);
+    o[0] = w[0], o[1] = w[1], o[2] = w[2], o[3] = w[3];
+  }
+}
+template <typename T, int V> __device__ __forceinline__ void stv(T* p, const float* v) {
+  if constexpr (V == 1) {
+    stf<T>(p, 0, v[0]);
+  } else if constexpr (sizeof(T) == 2) {
+    uint2 w;
+    w.x = pack_bf16x2(v[0], v[1]);
+    w.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(p) = w;
+  } else {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  }
+}
+
 // One residual step of a model with S parallel residual streams X [rows, S, W]
 // (fp32, updated in place).  With y (the previous sublayer's output):
 //     X_t <- sum_s mix[s, t] X_s + gain[t] * y          for every stream t
 // then, with read-in weights rin [S]:  u = sum_s rin[s] X_s  and
 //     out = u / sqrt(mean(u^2) + eps) * nw              (nw fp32 [W]; nw == null: out = u)
 // S = 1, mix = [1], gain = [1], rin = [1] is the ordinary pre-norm residual.
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) stream_step_kernel(float* __restrict__ X, const T* __restrict__ y,
                                                                int64_t y_stride, const float* __restrict__ mix,
                                                                const float* __restrict__ gain,
@@ -49,44 +74,63 @@ __global__ void __launch_bounds__(kThreads) stream_step_kernel(float* __restrict
   }
   __syncthreads();
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += kThreads) {
-    float v[kMaxStreams];
+  for (int c = threadIdx.x * V; c < W; c += kThreads * V) {
+    float v[kMaxStreams][V];
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s) v[s] = s < S ? x[(int64_t)s * W + c] : 0.f;
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < S) ldv<float, V>(x + (int64_t)s * W + c, v[s]);
     if (y) {
-      const float yv = ldf<T>(y, row * y_stride + c);
-      float n[kMaxStreams];
+      float yv[V], n[kMaxStreams][V];
+      ldv<T, V>(y + row * y_stride + c, yv);
 #pragma unroll
       for (int t = 0; t < kMaxStreams; ++t) {
-        float a = 0.f;
         if (t < S) {
 #pragma unroll
-          for (int s = 0; s < kMaxStreams; ++s)
-            if (s < S) a += s_mix[s * S + t] * v[s];
-          a += s_gain[t] * yv;
-          x[(int64_t)t * W + c] = a;
+          for (int e = 0; e < V; ++e) {
+            float a = s_gain[t] * yv[e];
+#pragma unroll
+            for (int s = 0; s < kMaxStreams; ++s)
+              if (s < S) a += s_mix[s * S + t] * v[s][e];
+            n[t][e] = a;
+          }
+          stv<float, V>(x + (int64_t)t * W + c, n[t]);
         }
-        n[t] = a;
       }
 #pragma unroll
-      for (int t = 0; t < kMaxStreams; ++t) v[t] = n[t];
+      for (int t = 0; t < kMaxStreams; ++t)
+        if (t < S) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[t][e] = n[t][e];
+        }
     }
     if (rin) {
-      float uu = 0.f;
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s)
-        if (s < S) uu += s_in[s] * v[s];
-      ss += uu * uu;
+      for (int e = 0; e < V; ++e) {
+        float uu = 0.f;
+#pragma unroll
+        for (int s = 0; s < kMaxStreams; ++s)
+          if (s < S) uu += s_in[s] * v[s][e];
+        ss += uu * uu;
+      }
     }
   }
   if (!rin) return;
   const float tot = block_reduce_sum(ss, red);
   const float r = nw ? rsqrtf(tot / (float)W + eps) : 1.f;
   // second pass: this thread re-reads the stream values it wrote itself
-  for (int c = threadIdx.x; c < W; c += kThreads) {
-    float uu = 0.f;
-    for (int s = 0; s < S; ++s) uu += s_in[s] * x[(int64_t)s * W + c];
-    stf<T>(out, row * out_stride + c, nw ? uu * r * nw[c] : uu);
+  for (int c = threadIdx.x * V; c < W; c += kThreads * V) {
+    float u[V], o[V], xv[V], wv[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) u[e] = 0.f;
+    for (int s = 0; s < S; ++s) {
+      ldv<float, V>(x + (int64_t)s * W + c, xv);
+#pragma unroll
+      for (int e = 0; e < V; ++e) u[e] += s_in[s] * xv[e];
+    }
+    if (nw) ldv<float, V>(nw + c, wv);
+#pragma unroll
+    for (int e = 0; e < V; ++e) o[e] = nw ? u[e] * r * wv[e] : u[e];
+    stv<T, V>(out + row * out_stride + c, o);
   }
 }
 
@@ -112,13 +156,17 @@ __device__ __forceinline__ float act_fn(float z, int act) {
 }
 
 // gu [rows, 2F] = [gate | up]  ->  out [rows, F] = act(gate) * up
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) glu_act_kernel(T* __restrict__ out, const T* __restrict__ gu, int F,
                                                            int64_t in_stride, int64_t out_stride, int act) {
   const int64_t r = blockIdx.y;
-  for (int c = blockIdx.x * kThreads + threadIdx.x; c < F; c += gridDim.x * kThreads) {
-    const float g = ldf<T>(gu, r * in_stride + c), u = ldf<T>(gu, r * in_stride + F + c);
-    stf<T>(out, r * out_stride + c, act_fn(g, act) * u);
+  for (int c = (blockIdx.x * kThreads + threadIdx.x) * V; c < F; c += gridDim.x * kThreads * V) {
+    float g[V], u[V], o[V];
+    ldv<T, V>(gu + r * in_stride + c, g);
+    ldv<T, V>(gu + r * in_stride + F + c, u);
+#pragma unroll
+    for (int e = 0; e < V; ++e) o[e] = act_fn(g[e], act) * u[e];
+    stv<T, V>(out + r * out_stride + c, o);
   }
 }
 
@@ -221,8 +269,16 @@ int dxm_stream_step(float* X, const void* y, int64_t y_stride, const float* mix,
   if (rows <= 0) return 0;
   if (y && (!mix || !gain)) return 2;
   if (rin && !out) return 3;
-  DISPATCH_T(f32, hipLaunchKernelGGL(stream_step_kernel<T>, dim3(rows), dim3(kThreads), 0, st, X, (const T*)y,
-                                     y_stride, mix, gain, rin, nw, eps, (T*)out, out_stride, S, W));
+  const int esz = f32 ? 4 : 2;
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)X % 16 == 0 &&
+                   (uintptr_t)y % (4 * esz) == 0 && (uintptr_t)out % (4 * esz) == 0 && (uintptr_t)nw % 16 == 0;
+  if (vec) {
+    DISPATCH_T(f32, hipLaunchKernelGGL((stream_step_kernel<T, 4>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)y,
+                                       y_stride, mix, gain, rin, nw, eps, (T*)out, out_stride, S, W));
+  } else {
+    DISPATCH_T(f32, hipLaunchKernelGGL((stream_step_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)y,
+                                       y_stride, mix, gain, rin, nw, eps, (T*)out, out_stride, S, W));
+  }
   DX_CHECK_LAUNCH();
   return 0;
 }
@@ -240,12 +296,22 @@ int dxm_glu_act(void* out, const void* gu, int rows, int F, int64_t in_stride, i
                 hipStream_t st) {
   if (rows <= 0 || F <= 0) return 0;
   if (act < 0 || act > 2) return 1;
-  const int gx = (F + kThreads - 1) / kThreads;
+  const int esz = f32 ? 4 : 2;
+  const bool vec = F % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)gu % (4 * esz) == 0 &&
+                   (uintptr_t)out % (4 * esz) == 0;
+  const int per = kThreads * (vec ? 4 : 1);
+  const int gx = (F + per - 1) / per;
   for (int r0 = 0; r0 < rows; r0 += 65535) {
     const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
-    DISPATCH_T(f32, hipLaunchKernelGGL(glu_act_kernel<T>, dim3(gx, nr), dim3(kThreads), 0, st,
-                                       (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
-                                       out_stride, act));
+    if (vec) {
+      DISPATCH_T(f32, hipLaunchKernelGGL((glu_act_kernel<T, 4>), dim3(gx, nr), dim3(kThreads), 0, st,
+                                         (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
+                                         out_stride, act));
+    } else {
+      DISPATCH_T(f32, hipLaunchKernelGGL((glu_act_kernel<T, 1>), dim3(gx, nr), dim3(kThreads), 0, st,
+                                         (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
+                                         out_stride, act));
+    }
   }
   DX_CHECK_LAUNCH();
   return 0;

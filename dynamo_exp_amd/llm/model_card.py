@@ -63,7 +63,7 @@ class ModelDeploymentCard:
         """From an HF directory (config + tokenizer files) or a preset name."""
         files = {}
         if os.path.isdir(model):
-            cfg = ModelConfig.from_hf_dir(model)
+            cfg = get_config(model)  # the config file names its architecture (Llama / LLaVA / layer-listed)
             for f in ("config.json", "tokenizer.json", "tokenizer_config.json", "generation_config.json"):
                 p = os.path.join(model, f)
                 if os.path.exists(p):
@@ -78,11 +78,11 @@ class ModelDeploymentCard:
                    prompt_context=["llama3_date_time"] if "llama" in cfg.architecture.lower() else [])
 
     def model_config(self) -> ModelConfig:
-        if "architectures" in self.model_info:
+        if "architectures" in self.model_info or "architecture" in self.model_info:
             d = tempfile.mkdtemp(prefix="dx_mdc_cfg_")
             with open(os.path.join(d, "config.json"), "w") as f:
                 json.dump(self.model_info, f)
-            return ModelConfig.from_hf_dir(d)
+            return get_config(d)
         return ModelConfig.from_dict(self.model_info)
 
     def local_dir(self) -> str | None:
