@@ -196,7 +196,8 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
     if (nv <= 1) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 1>), grid, dim3(64), lds, st, b);
     else if (nv <= 2) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 2>), grid, dim3(64), lds, st, b);
     else if (nv <= 4) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 4>), grid, dim3(64), lds, st, b);
-    else hipLaunchKernelGGL((row_attention_kernel<T, OutT, 8>), grid, dim3(64), lds, st, b);
+    else if (nv <= 8) hipLaunchKernelGGL((row_attention_kernel<T, OutT, 8>), grid, dim3(64), lds, st, b);
+    else hipLaunchKernelGGL((row_attention_kernel<T, OutT, 16>), grid, dim3(64), lds, st, b);
     if (a.parts > 1)
       hipLaunchKernelGGL((merge_parts_kernel<OutT>), dim3((unsigned)nr * a.n_qh), dim3(64), 0, st, (OutT*)b.out, b.ws,
                          a.parts, a.dv);
@@ -213,7 +214,7 @@ extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_
                                  int size, int parts, int f32, int out_f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group) return 1;
-  if (d < 1 || dv < 1 || dv > 512 || d > 8192) return 2;
+  if (d < 1 || dv < 1 || dv > 1024 || d > 8192) return 2;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535 || n_qh > 65535) return 3;
   if (parts > 1 && !ws) return 4;
   RowAttnArgs a{q, q_stride, kc, vc, out, ws, pos, seq, bt, bt_stride, bs, n_qh, maps, group,

@@ -235,20 +235,29 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
       i16x4 Ph[2][4], Pl[2][4];
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb) {
+        // scale > 0 (checked on the host): the row maximum is taken over the raw sums and
+        // scaled once, and the scale rides in the exponent's fma
         float mloc = -INFINITY;
+        if (full) {
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
+          for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int kj = kt + kb * 16 + 4 * g4 + i;
-            const bool vis = full || (okrow[qb] && kj >= lrow[qb] && kj <= prow[qb]);
-            const float s = vis ? S[qb][kb][i] * sc2 : -INFINITY;  // log2 units
-            S[qb][kb][i] = s;
-            mloc = fmaxf(mloc, s);
-          }
+            for (int i = 0; i < 4; ++i) mloc = fmaxf(mloc, S[qb][kb][i]);
+        } else {
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int kj = kt + kb * 16 + 4 * g4 + i;
+              const bool vis = okrow[qb] && kj >= lrow[qb] && kj <= prow[qb];
+              const float s = vis ? S[qb][kb][i] : -INFINITY;
+              S[qb][kb][i] = s;
+              mloc = fmaxf(mloc, s);
+            }
+        }
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-        const float mn = fmaxf(mx[qb], mloc);
+        const float mn = fmaxf(mx[qb], mloc * sc2);  // log2 units
         const float mu = mn == -INFINITY ? 0.f : mn;  // a row that sees nothing in this tile
         const float alpha = fast_exp2(mx[qb] - mu);
         mx[qb] = mn;
@@ -258,7 +267,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
           float p[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            p[i] = fast_exp2(S[qb][kb][i] - mu);
+            p[i] = fast_exp2(fmaf(S[qb][kb][i], sc2, -mu));
             add += p[i];
           }
           const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
@@ -267,9 +276,14 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
           Ph[qb][kb] = __builtin_bit_cast(i16x4, uint2{h01, h23});
           Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
         }
-        lsum[qb] = lsum[qb] * alpha + add;
+        // the running maximum of no row of the wave moved: nothing to rescale
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+          lsum[qb] = lsum[qb] * alpha + add;
 #pragma unroll
-        for (int cb = 0; cb < DVB; ++cb) O[qb][cb] *= alpha;
+          for (int cb = 0; cb < DVB; ++cb) O[qb][cb] *= alpha;
+        } else {
+          lsum[qb] += add;
+        }
       }
 #pragma unroll
       for (int kp = 0; kp < 2; ++kp) {  // 32 keys per MFMA: key blocks 2 kp and 2 kp + 1
@@ -529,7 +543,7 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
                        hipStream_t st) {
   if (n_tiles <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
-  if (mask < 0 || mask > 2 || (mask && size < 1)) return 3;
+  if (mask < 0 || mask > 2 || (mask && size < 1) || !(scale > 0.f)) return 3;
   if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 8) return 4;
   TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
              tiles, n_qh, maps, group, Wk, Wv, scale, mask, size};

@@ -222,7 +222,7 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     does not apply) on the row kernel.  Same arguments and result as
     row_attention."""
     T = q.shape[0]
-    if not tile_attention_ok(q, d, dv):
+    if not tile_attention_ok(q, d, dv) or not scale > 0:  # the matrix-core kernels fold a positive scale
         return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
                              mask, size, parts, out_f32)
     if tiles is None:

@@ -70,6 +70,9 @@ CONFIGS = {
     "ones": lambda: config([att(H=4, G=1, d=8, every=1), lat(H=2, d=8, dv=8, r=8, window=1),
                             dif(H=2, G=1, d=8, dv=8, chunk=1, diff=0.0)], width=32, streams=1,
                            loop={"start": 1, "stop": 2, "times": 1}),
+    # nothing divides by 4 or 8: width, vocabulary, feed-forward and head widths on the scalar paths, five streams
+    "odd": lambda: config([att(H=3, G=1, d=18, mlp=50), lat(H=3, d=10, dv=14, r=38, window=7, mlp=34),
+                           dif(H=2, G=2, d=6, dv=22, chunk=5, mlp=None)], width=102, vocab=101, streams=5),
     # head widths the matrix-core prefill kernel serves (bf16 on the GPU)
     "tiles": lambda: config([att(H=4, G=2, d=32, every=16), lat(H=2, d=16, dv=32, r=48, window=20),
                              dif(H=2, G=1, d=64, dv=128, chunk=24), att(H=2, G=1, d=64, coef=0.0)], width=64,
