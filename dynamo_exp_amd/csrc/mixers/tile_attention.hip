@@ -11,9 +11,10 @@
 //     O^T = V^T P^T   A = V^T (LDS),    B = P^T = the S^T accumulator itself
 // (v_mfma_f32_16x16x16_bf16: lane l holds column l % 16 and rows 4 (l / 16)
 // .. + 3 of C, which is exactly the B layout of the next product).  Scores are
-// the exact fp32 sums of bf16 products; the softmax is fp32; the weights enter
-// the second product as a bf16 pair hi + lo (two MFMAs), which keeps 16
-// mantissa bits of every weight instead of 8.
+// the exact fp32 sums of bf16 products; the softmax is fp32.  With bf16 output
+// the weights enter the second product as bf16, like the other bf16
+// activations; with fp32 output (and in the decode kernel) as a bf16 pair
+// hi + lo (two MFMAs), which keeps 16 mantissa bits of every weight.
 //
 // Masks are evaluated per element in sequence positions: causal, sliding
 // window (p - size < j <= p) and chunked (floor(j / size) == floor(p / size)),
@@ -150,6 +151,9 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* o, f32x4 v) {
 template <int DB, int DVB, typename OutT>
 __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_kernel(TileArgs a) {
   constexpr int d = DB * 16, dv = DVB * 16, ks_stride = d + 8;
+  // fp32 output (the two-map layers, whose a1 - lambda a2 amplifies errors): the weights enter
+  // the second product as hi + lo; bf16 output: as one bf16, like every other bf16 activation
+  constexpr bool kHiLo = sizeof(OutT) == 4;
   constexpr bool X32 = DB % 2 == 0;  // d a multiple of 32: the K = 32 MFMA for the scores too
   constexpr int DB2 = X32 ? DB / 2 : 1;
   extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
@@ -271,10 +275,12 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
             add += p[i];
           }
           const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
-          const uint32_t l01 = pack_bf16x2(p[0] - bf16lo(h01), p[1] - bf16hi(h01));
-          const uint32_t l23 = pack_bf16x2(p[2] - bf16lo(h23), p[3] - bf16hi(h23));
           Ph[qb][kb] = __builtin_bit_cast(i16x4, uint2{h01, h23});
-          Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
+          if constexpr (kHiLo) {
+            const uint32_t l01 = pack_bf16x2(p[0] - bf16lo(h01), p[1] - bf16hi(h01));
+            const uint32_t l23 = pack_bf16x2(p[2] - bf16lo(h23), p[3] - bf16hi(h23));
+            Pl[qb][kb] = __builtin_bit_cast(i16x4, uint2{l01, l23});
+          }
         }
         // the running maximum of no row of the wave moved: nothing to rescale
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
@@ -291,7 +297,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
           Bh[qb] = pair8(Ph[qb][2 * kp], Ph[qb][2 * kp + 1]);
-          Bl[qb] = pair8(Pl[qb][2 * kp], Pl[qb][2 * kp + 1]);
+          if constexpr (kHiLo) Bl[qb] = pair8(Pl[qb][2 * kp], Pl[qb][2 * kp + 1]);
         }
 #pragma unroll
         for (int cb = 0; cb < DVB; ++cb) {
@@ -300,7 +306,7 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
             O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, Bh[qb], O[qb][cb], 0, 0, 0);
-            O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, Bl[qb], O[qb][cb], 0, 0, 0);
+            if constexpr (kHiLo) O[qb][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, Bl[qb], O[qb][cb], 0, 0, 0);
           }
         }
       }
