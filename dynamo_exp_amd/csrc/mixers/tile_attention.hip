@@ -78,6 +78,7 @@ struct TileStage {
     return (int64_t)bt[u / b] * bs + u % b;
   }
 
+  template <bool DoK = true, bool DoV = true>
   __device__ __forceinline__ void fetch(const bf16_t* kc, const bf16_t* vc, const int* bt, int bs, int Wk, int Wv,
                                         int kt, int hi, int tid) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -86,7 +87,7 @@ struct TileStage {
     // global round trip in front of each of them, and the loads retire in order.
     const int mine = kt + (tid & 63) <= hi ? (int)slot_of(bt, bs, kt + (tid & 63)) : -1;
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) {
+    for (int i = 0; i < (DoK ? kPer : 0); ++i) {
       const int it = tid + i * NT;
       const int key = it / (d / 8), ch = it % (d / 8);
       const int64_t slot = __shfl(mine, key & 63, 64);
@@ -94,7 +95,7 @@ struct TileStage {
       kr[i] = ok ? *reinterpret_cast<const u32x4*>(kc + slot * Wk + ch * 8) : zero;
     }
 #pragma unroll
-    for (int i = 0; i < vPer; ++i) {
+    for (int i = 0; i < (DoV ? vPer : 0); ++i) {
       const int it = tid + i * NT;
       const int kg = it / (dv / 8), ch = it % (dv / 8);
 #pragma unroll
@@ -106,14 +107,15 @@ struct TileStage {
     }
   }
 
+  template <bool DoK = true, bool DoV = true>
   __device__ __forceinline__ void commit(bf16_t* Ks, bf16_t* Vt, int tid) const {
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) {
+    for (int i = 0; i < (DoK ? kPer : 0); ++i) {
       const int it = tid + i * NT;
       if (it < kItems) *reinterpret_cast<u32x4*>(Ks + (it / (d / 8)) * ks_stride + (it % (d / 8)) * 8) = kr[i];
     }
 #pragma unroll
-    for (int i = 0; i < vPer; ++i) {
+    for (int i = 0; i < (DoV ? vPer : 0); ++i) {
       const int it = tid + i * NT;
       if (it >= vItems) continue;
       const int kg = it / (dv / 8), ch = it % (dv / 8);
@@ -392,13 +394,23 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
 #pragma unroll
     for (int cb = 0; cb < DVB; ++cb) O[qb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+  // wide heads: a whole tile in flight would not fit the register file beside the
+  // accumulators, so K and V are staged one after the other and nothing is prefetched
+  constexpr bool kWide = DB + DVB > 16;
   TileStage<d, dv, 64> stage;
-  if (t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, lo + t0 * kKeys, p, lane);
+  if (!kWide && t0 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, lo + t0 * kKeys, p, lane);
   for (int t = t0; t < t1; ++t) {
     const int kt = lo + t * kKeys;
-    stage.commit(Ks, Vt, lane);
+    if constexpr (kWide) {
+      stage.template fetch<true, false>(kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+      stage.template commit<true, false>(Ks, Vt, lane);
+      stage.template fetch<false, true>(kc, vc, bt, a.bs, a.Wk, a.Wv, kt, p, lane);
+      stage.template commit<false, true>(Ks, Vt, lane);
+    } else {
+      stage.commit(Ks, Vt, lane);
+    }
     __syncthreads();
-    if (t + 1 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, p, lane);
+    if (!kWide && t + 1 < t1) stage.fetch(kc, vc, bt, a.bs, a.Wk, a.Wv, kt + kKeys, p, lane);
     f32x4 S[QB][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -484,8 +496,8 @@ template <int DB, int DVB>
 int launch_group(const GroupArgs& a0, int rows, hipStream_t st) {
   const size_t lds = (size_t)(kKeys * (DB * 16 + 8) + DVB * 16 * kVtStride) * sizeof(bf16_t);
   GroupArgs a = a0;
-  const bool two = a.group > 16;
-  a.chunks = two ? (a.group + 31) / 32 : 1;
+  const bool two = a.group > 16 && DB + DVB <= 16;  // two head blocks per wave only where the registers hold them
+  a.chunks = two ? (a.group + 31) / 32 : (a.group + 15) / 16;
   auto k1 = group_decode_kernel<DB, DVB, 1>;
   auto k2 = group_decode_kernel<DB, DVB, 2>;
   if (lds > 48 * 1024) {

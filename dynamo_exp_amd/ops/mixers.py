@@ -29,7 +29,7 @@ MAX_STREAMS = 8
 # row attention: aim for this many waves per launch, never split a row's keys
 # into parts shorter than ROW_MIN_PART
 ROW_TARGET_WAVES = 2048
-ROW_MIN_PART = 256
+ROW_MIN_PART = 128
 
 
 def _m():
