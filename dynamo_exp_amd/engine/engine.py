@@ -341,7 +341,7 @@ class LLMEngine:
 
         batch = self.scheduler.schedule_forced(entries, new_request)
         self.last_batch = batch
-        logits = self.runner.score(batch)
+        logits = self.runner.score(batch) if batch.requests else []  # a step may only end requests
         self.scheduler.update_forced(batch, list(end or []))
         for rid in end or []:
             self.requests.pop(rid, None)
