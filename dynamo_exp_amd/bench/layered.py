@@ -148,6 +148,50 @@ def attention_kernels(s: dict, L: int, B: int) -> dict:
     return res
 
 
+def rowwise_kernels(s: dict, T: int) -> dict:
+    """The memory-bound row kernels alone at T rows, in TB/s of the bytes each
+    has to move: residual step + norm, gated activation, head prep + cache write,
+    each beside Llama's counterpart."""
+    W, ff, H, G, d = s["W"], s["ff"], s["H"], s["G"], s["d"]
+    dev, dt, S, bs = "cuda", torch.bfloat16, 4, 64
+    res = {}
+
+    def put(name, us, byts):
+        res[name] = {"us": round(us, 1), "TB/s": round(byts / us / 1e6, 2)}
+
+    X = torch.randn(T, S, W, device=dev)
+    y = torch.randn(T, W, device=dev, dtype=dt)
+    mixw = torch.eye(S, device=dev) + 0.01
+    ones = torch.ones(S, device=dev)
+    nw = torch.ones(W, device=dev)
+    put("bekulix_stream_step", _timed(lambda: mx.stream_step(X, y, mixw, ones, ones, nw, 1e-6, dt)),
+        T * W * (2 * S * 4 + 2 + 2))  # streams read + written (fp32), y in, normed row out
+    h = torch.randn(T, W, device=dev, dtype=dt)
+    r = torch.randn(T, W, device=dev, dtype=dt)
+    w16 = torch.ones(W, device=dev, dtype=dt)
+    put("llama_add_rmsnorm", _timed(lambda: ops.add_rmsnorm(h, r, w16, 1e-6)), T * W * 2 * 4)
+    gu = torch.randn(T, 2 * ff, device=dev, dtype=dt)
+    put("bekulix_glu_act", _timed(lambda: mx.glu_act(gu, "relu")), T * ff * 2 * 3)
+    put("llama_silu_and_mul", _timed(lambda: ops.silu_and_mul(gu)), T * ff * 2 * 3)
+    nb = T // bs + 1
+    p = torch.randn(T, (H + G) * d, device=dev, dtype=dt)
+    pos = torch.arange(T, device=dev)
+    kc = torch.zeros(nb * bs, G * d, device=dev, dtype=dt)
+    vc = torch.zeros_like(kc)
+    qn = torch.ones(d, device=dev)
+    put("bekulix_headprep_cache", _timed(lambda: mx.headprep_cache(p, pos, pos, H, G, d, H * d, qn, qn, 1e-6, (0.1, 4096),
+                                                                   kc, vc, v_mode=1)),
+        T * d * 2 * (2 * H + 3 * G))  # q read + written, k read, K and V rows written
+    qkv = torch.randn(T, (H + 2 * G) * d, device=dev, dtype=dt)
+    from ..ops import reference as ref
+    cs = ref.rope_cos_sin(d, T + 1, 500000.0, None).to(dev)
+    kl = torch.zeros(nb, G, bs, d, device=dev, dtype=dt)
+    vl = torch.zeros_like(kl)
+    put("llama_rope_cache", _timed(lambda: ops.rope_cache(qkv, pos, cs, pos, kl, vl, H, G, d, bs)),
+        T * d * 2 * (2 * H + 4 * G))
+    return res
+
+
 def run_layered_compare(args, dev) -> dict:
     isl, osl = min(args.isl, 2048), min(args.osl, 64)
     sizes = {}
@@ -157,6 +201,7 @@ def run_layered_compare(args, dev) -> dict:
         row["bekulix"] = engine_throughput(bek, dev, isl, osl, 4, 64, args.seed)
         row["llama"] = engine_throughput(lla, dev, isl, osl, 4, 64, args.seed)
         row["attention_kernels"] = attention_kernels(s, 4096, 64)
+        row["rowwise_kernels"] = rowwise_kernels(s, 8192)
         sizes[name] = row
     return {"metric": "layer-listed model (Bekulix) beside Llama at equal layer sizes: engine prefill / decode "
                       "tokens/s and attention kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",

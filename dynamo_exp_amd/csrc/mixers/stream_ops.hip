@@ -47,6 +47,16 @@ template <typename T, int V> __device__ __forceinline__ void stv(T* p, const flo
   }
 }
 
+template <typename T, int V> __device__ __forceinline__ void cpv(T* dst, const T* src) {  // raw copy of V elements
+  if constexpr (V == 1) {
+    dst[0] = src[0];
+  } else if constexpr (sizeof(T) == 2) {
+    *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(src);
+  } else {
+    *reinterpret_cast<f32x4*>(dst) = *reinterpret_cast<const f32x4*>(src);
+  }
+}
+
 // One residual step of a model with S parallel residual streams X [rows, S, W]
 // (fp32, updated in place).  With y (the previous sublayer's output):
 //     X_t <- sum_s mix[s, t] X_s + gain[t] * y          for every stream t
@@ -177,14 +187,18 @@ __global__ void __launch_bounds__(kThreads) glu_act_kernel(T* __restrict__ out, 
 //      the K cache row of the token's slot (kc [slots, n_k * d])
 //   v: v_mode 0: no V cache (V is the K cache); 1: the k section as projected
 //      (before its norm) is the value; 2: v_w columns at v_off are the value
-// slot < 0: nothing is cached for the row.  One wave per vector.
-template <typename T>
+// slot < 0: nothing is cached for the row.
+template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
     T* __restrict__ x, int64_t x_stride, const int64_t* __restrict__ pos, const int64_t* __restrict__ slots,
     int n_q, int n_k, int d, int k_off, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
-    float temp_coef, double temp_every, T* __restrict__ kc, T* __restrict__ vc, int v_mode, int v_off, int v_w) {
+    float temp_coef, double temp_every, T* __restrict__ kc, T* __restrict__ vc, int v_mode, int v_off, int v_w,
+    int lpv) {
+  // lpv lanes (a power of two) share one head vector, so a wave works on 64 / lpv
+  // vectors at once and their loads overlap; the sum of squares is reduced inside the group
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = kThreads / 64;
+  const int per_wave = 64 / lpv, grp = lane / lpv, gl = lane - grp * lpv;
   T* row = x + t * x_stride;
   const int64_t slot = slots[t];
   const int k_w = n_k * d;
@@ -194,7 +208,7 @@ __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
     gain = 1.f + temp_coef * logf((float)k + 1.f);
   }
   const bool q_work = qw != nullptr || temp_coef != 0.f;
-  for (int v = wid; v < n_q + n_k; v += nw) {
+  for (int v = wid * per_wave + grp; v < n_q + n_k; v += nw * per_wave) {
     const bool is_q = v < n_q;
     if (is_q && !q_work) continue;
     if (!is_q && slot < 0) continue;
@@ -203,28 +217,32 @@ __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
     float r = 1.f;
     if (w) {
       float ss = 0.f;
-      for (int e = lane; e < d; e += 64) {
-        const float a = ldf<T>(src, e);
-        ss += a * a;
+      for (int e = gl * V; e < d; e += lpv * V) {
+        float a[V];
+        ldv<T, V>(src + e, a);
+#pragma unroll
+        for (int i = 0; i < V; ++i) ss += a[i] * a[i];
       }
-      r = rsqrtf(wave_reduce_sum(ss) / (float)d + eps);
+      for (int o = lpv >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      r = rsqrtf(ss / (float)d + eps);
     }
-    if (is_q) {
-      for (int e = lane; e < d; e += 64) stf<T>(src, e, ldf<T>(src, e) * (w ? r * w[e] : 1.f) * gain);
-    } else {
-      T* kd = kc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d;
-      T* vd = v_mode == 1 ? vc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d : nullptr;
-      for (int e = lane; e < d; e += 64) {
-        const float a = ldf<T>(src, e);
-        if (vd) vd[e] = src[e];
-        stf<T>(kd, e, w ? a * r * w[e] : a);
-      }
+    T* kd = is_q ? src : kc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d;
+    T* vd = (!is_q && v_mode == 1) ? vc + slot * (int64_t)k_w + (int64_t)(v - n_q) * d : nullptr;
+    const float g = is_q ? gain : 1.f;
+    for (int e = gl * V; e < d; e += lpv * V) {
+      float a[V], wv[V];
+      ldv<T, V>(src + e, a);
+      if (vd) cpv<T, V>(vd + e, src + e);
+      if (w) ldv<float, V>(w + e, wv);
+#pragma unroll
+      for (int i = 0; i < V; ++i) a[i] = a[i] * (w ? r * wv[i] : 1.f) * g;
+      stv<T, V>(kd + e, a);
     }
   }
   if (v_mode == 2 && slot >= 0) {
     const T* vs = row + v_off;
     T* vd = vc + slot * (int64_t)v_w;
-    for (int e = threadIdx.x; e < v_w; e += kThreads) vd[e] = vs[e];
+    for (int e = threadIdx.x * V; e < v_w; e += kThreads * V) cpv<T, V>(vd + e, vs + e);
   }
 }
 
@@ -326,9 +344,23 @@ int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int6
   if (n_k > 0 && !kc) return 2;
   if (v_mode != 0 && !vc) return 3;
   if (temp_coef != 0.f && !(temp_every > 0)) return 4;
-  DISPATCH_T(f32, hipLaunchKernelGGL(headprep_cache_kernel<T>, dim3(rows), dim3(kThreads), 0, st, (T*)x, x_stride, pos,
-                                     slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every, (T*)kc, (T*)vc,
-                                     v_mode, v_off, v_w));
+  const int esz = f32 ? 4 : 2;
+  const bool vec = d % 4 == 0 && k_off % 4 == 0 && x_stride % 4 == 0 && v_off % 4 == 0 && v_w % 4 == 0 &&
+                   (uintptr_t)x % (4 * esz) == 0 && (uintptr_t)kc % (4 * esz) == 0 && (uintptr_t)vc % (4 * esz) == 0 &&
+                   (uintptr_t)qw % 16 == 0 && (uintptr_t)kw % 16 == 0;
+  // lanes per head vector: about two chunks of V elements per lane
+  const int chunks = (d + (vec ? 4 : 1) - 1) / (vec ? 4 : 1);
+  int lpv = 1;
+  while (lpv < 64 && lpv * 2 < chunks) lpv <<= 1;
+  if (vec) {
+    DISPATCH_T(f32, hipLaunchKernelGGL((headprep_cache_kernel<T, 4>), dim3(rows), dim3(kThreads), 0, st, (T*)x,
+                                       x_stride, pos, slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every,
+                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, lpv));
+  } else {
+    DISPATCH_T(f32, hipLaunchKernelGGL((headprep_cache_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, st, (T*)x,
+                                       x_stride, pos, slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every,
+                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, lpv));
+  }
   DX_CHECK_LAUNCH();
   return 0;
 }
