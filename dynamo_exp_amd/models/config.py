@@ -148,6 +148,8 @@ class LayeredConfig:
     loop: dict | None = None  # {"start", "stop", "times"}
     rms_norm_eps: float = 1e-6
     streams: int | None = None  # parallel residual streams (None: one plain residual)
+    token_side: dict | None = None  # {"dim"}: per-layer token input (a slice of a second embedding per layer)
+    learned_positions: bool = False  # a learned vector per position is added to the embedding
     max_position_embeddings: int = 1 << 20
     tie_word_embeddings: bool = False
     bos_token_id: int = 0
@@ -173,6 +175,8 @@ class LayeredConfig:
     def num_params(self) -> int:
         W = self.hidden_size
         n = 2 * self.vocab_size * W + W
+        if self.architecture == "Bolinex":
+            return n + self._bolinex_params()
         for L in self.layers:
             m, t = L["mixer"], L["type"]
             H, d, dv = m["heads"], m["dim"], m["vdim"]
@@ -187,16 +191,40 @@ class LayeredConfig:
                 n += 3 * W * L["mlp"]["ff"]
         return n
 
+    def _bolinex_params(self) -> int:
+        W = self.hidden_size
+        n = W  # norm biases ride with the weights: final bias
+        if self.learned_positions:
+            n += self.max_position_embeddings * W
+        side = (self.token_side or {}).get("dim", 0)
+        n += self.vocab_size * side * len(self.layers)
+        for L in self.layers:
+            m = L["mixer"]
+            H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            n += 2 * W + (H * d + G * d + G * dv + H * dv) * W + W * H * dv + 2 * H + 1
+            mlp = L.get("mlp")
+            if mlp and mlp["kind"] == "dense":
+                n += 2 * W * mlp["ff"]
+            elif mlp:
+                E = mlp["router"]["experts"]
+                n += E * 3 * W * mlp["expert"]["ff"] + E * W + E
+                if mlp.get("shared"):
+                    n += 3 * W * mlp["shared"]["ff"]
+            n += 2 * W * side + (W if side else 0)
+        return n
+
     def to_dict(self) -> dict:
         return dataclasses.asdict(self)
 
     @classmethod
     def from_dict(cls, c: dict, name: str = "layered") -> "LayeredConfig":
         """From the checkpoint's config.json."""
+        maxpos = c.get("max_positions", c.get("max_position_embeddings"))
         return cls(name=name, architecture=c["architecture"], vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
                    layers=list(c["layers"]), loop=c.get("loop"), rms_norm_eps=float(c["norm"]["eps"]),
-                   streams=c.get("streams"),
-                   max_position_embeddings=int(c.get("max_position_embeddings", 1 << 20)),
+                   streams=c.get("streams"), token_side=c.get("token_side"),
+                   learned_positions="max_positions" in c,
+                   max_position_embeddings=int(maxpos) if maxpos else 1 << 20,
                    eos_token_id=list(c.get("eos_token_id", [])))
 
     def write_hf_config(self, path: str) -> None:
@@ -207,12 +235,16 @@ class LayeredConfig:
             d["loop"] = self.loop
         if self.streams:
             d["streams"] = self.streams
+        if self.token_side:
+            d["token_side"] = self.token_side
+        if self.learned_positions:
+            d["max_positions"] = self.max_position_embeddings
         with open(os.path.join(path, "config.json"), "w") as f:
             json.dump(d, f, indent=1)
 
 
 # config.json `architecture` values served by LayeredConfig
-LAYERED_ARCHITECTURES = ("Bekulix",)
+LAYERED_ARCHITECTURES = ("Bekulix", "Bolinex")
 
 
 def _bekulix_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, window, chunk, vocab=32000, streams=4):
@@ -230,6 +262,24 @@ def _bekulix_preset(name, W, ff, n_layers, heads, kv_heads, d, rank, window, chu
     cyc = [att, lat, att, dif]
     return LayeredConfig(name=name, vocab_size=vocab, hidden_size=W, layers=[dict(cyc[i % 4]) for i in range(n_layers)],
                          streams=streams)
+
+
+def _bolinex_preset(name, W, ff, n_layers, heads, kv_heads, d, window, experts=0, top=2, expert_ff=0, shared_ff=0,
+                    groups=(1, 1), side=0, vocab=32000, max_positions=8192, softcap=30.0):
+    """A Bolinex stack at a real model's layer sizes: windowed grouped-query
+    attention with a tanh score cap, a distance penalty, value mixing and an
+    output gate, in parallel with a dense (relu squared) feed-forward or, on
+    every second layer when `experts` > 0, a routed mixture of experts."""
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": softcap,
+             "mask": {"size": window}, "v_mix": True}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff} if shared_ff else None,
+           "router": {"experts": experts, "top": top, "groups": {"count": groups[0], "keep": groups[1]}}}
+    layers = [{"type": "attention", "mixer": dict(mixer), "mlp": dict(moe if experts and i % 2 else dense)}
+              for i in range(n_layers)]
+    return LayeredConfig(name=name, architecture="Bolinex", vocab_size=vocab, hidden_size=W, layers=layers,
+                         rms_norm_eps=1e-5, token_side={"dim": side} if side else None, learned_positions=True,
+                         max_position_embeddings=max_positions)
 
 
 # CLIP ViT-L/14 at 336 px, the LLaVA-1.5 vision tower; features from the
@@ -287,6 +337,14 @@ PRESETS: dict[str, ModelConfig] = {
 PRESETS["bekulix-tiny"] = _bekulix_preset("bekulix-tiny", 256, 512, 4, 4, 2, 64, 64, 48, 96, vocab=512)
 # Llama-3-8B's layer sizes (width 4096, ff 14336, 32 x 128 heads, 8 KV heads), 8 layers
 PRESETS["bekulix-8b-shapes"] = _bekulix_preset("bekulix-8b-shapes", 4096, 14336, 8, 32, 8, 128, 512, 1024, 2048,
+                                               vocab=128256)
+
+
+PRESETS["bolinex-tiny"] = _bolinex_preset("bolinex-tiny", 256, 512, 4, 4, 2, 64, 96, experts=8, top=2, expert_ff=128,
+                                          shared_ff=128, groups=(4, 2), side=32, vocab=512, max_positions=4096)
+# Llama-3-8B's layer sizes, 8 layers, every second feed-forward 16 experts of a quarter of the dense width
+PRESETS["bolinex-8b-shapes"] = _bolinex_preset("bolinex-8b-shapes", 4096, 14336, 8, 32, 8, 128, 1024, experts=16,
+                                               top=2, expert_ff=3584, shared_ff=3584, groups=(4, 2), side=256,
                                                vocab=128256)
 
 

@@ -24,11 +24,18 @@ def _bekulix():
     return BekulixForCausalLM
 
 
+def _bolinex():
+    from .bolinex import BolinexForCausalLM
+
+    return BolinexForCausalLM
+
+
 # architecture -> (class loader, activation dtypes the class has kernels for)
 MODEL_REGISTRY = {
     "LlamaForCausalLM": (_llama, ("bfloat16",)),
     "LlavaForConditionalGeneration": (_llama, ("bfloat16",)),
     "Bekulix": (_bekulix, ("bfloat16", "float32")),
+    "Bolinex": (_bolinex, ("bfloat16", "float32")),
 }
 
 

@@ -24,7 +24,8 @@ import torch
 from .. import _native
 
 MASKS = {"causal": 0, "window": 1, "chunk": 2}
-ACTS = {"relu": 0, "silu": 1, "gelu_tanh": 2}
+ACTS = {"relu": 0, "silu": 1, "gelu_tanh": 2, "sigmoid": 3, "relu2": 4}
+NORMS = {None: 0, "rms": 1, "layer": 2}
 MAX_STREAMS = 8
 # row attention: aim for this many waves per launch, never split a row's keys
 # into parts shorter than ROW_MIN_PART
@@ -58,16 +59,87 @@ def _fp32_param(t: torch.Tensor | None, name: str):
 
 
 # ----------------------------------------------------------------- residual streams
-def embed_streams(ids: torch.Tensor, table: torch.Tensor, n_streams: int) -> torch.Tensor:
-    """X [T, S, W] fp32 with every stream equal to table[ids]."""
+def embed_streams(ids: torch.Tensor, table: torch.Tensor, n_streams: int, pos_table: torch.Tensor | None = None,
+                  positions: torch.Tensor | None = None) -> torch.Tensor:
+    """X [T, S, W] fp32 with every stream equal to table[ids], plus the learned
+    position vector pos_table[positions] when a table of them is given (the
+    sum is formed in fp32)."""
     T = ids.shape[0]
     V, W = table.shape
+    if pos_table is not None and (positions is None or pos_table.shape[1] != W or pos_table.dtype != table.dtype):
+        raise ValueError("embed_streams: position table of the embedding's width and dtype, with positions")
     if not table.is_cuda:
-        return table[ids].float()[:, None, :].repeat(1, n_streams, 1).contiguous()
+        x = table[ids].float()
+        if pos_table is not None:
+            x = x + pos_table[positions].float()
+        return x[:, None, :].repeat(1, n_streams, 1).contiguous()
     X = torch.empty((T, n_streams, W), dtype=torch.float32, device=table.device)
     ids = ids if ids.dtype == torch.int64 else ids.long()
-    _m().embed_streams(X.data_ptr(), table.data_ptr(), ids.data_ptr(), T, n_streams, W, V, _f32(table), _stream())
+    if pos_table is not None and (positions.dtype != torch.int64 or not pos_table.is_contiguous()):
+        raise TypeError("embed_streams: int64 positions, contiguous position table")
+    _m().embed_streams(X.data_ptr(), table.data_ptr(), ids.data_ptr(), T, n_streams, W, V, _ptr(pos_table),
+                       _ptr(positions) if pos_table is not None else 0,
+                       pos_table.shape[0] if pos_table is not None else 0, _f32(table), _stream())
     return X
+
+
+def gather_rows(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """table[ids] in the table's dtype (rows outside the table read as zeros)."""
+    if not table.is_cuda:
+        return table[ids]
+    T, (V, W) = ids.shape[0], table.shape
+    out = torch.empty((T, W), dtype=table.dtype, device=table.device)
+    ids = ids if ids.dtype == torch.int64 else ids.long()
+    _m().gather_rows(out.data_ptr(), table.data_ptr(), ids.data_ptr(), T, W, V, _f32(table), _stream())
+    return out
+
+
+def residual_step(X: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tensor | None = None,
+                  c: torch.Tensor | None = None, c_w: torch.Tensor | None = None, eps: float = 1e-6,
+                  norm: str | None = None, norm_w: torch.Tensor | None = None, norm_b: torch.Tensor | None = None,
+                  out_dtype: torch.dtype = torch.bfloat16, want_cast: bool = False):
+    """One step of a single fp32 residual X [T, W], in place:
+        X <- X + a + b + c / sqrt(mean(c^2) + eps) * c_w        (each addend optional)
+    then, returned as (normed, cast):
+        normed = norm(X) in out_dtype: 'rms'  X / sqrt(mean(X^2) + eps) * norm_w,
+                                       'layer' (X - mean) / sqrt(var + eps) * norm_w + norm_b, None: nothing;
+        cast   = X in out_dtype when want_cast.
+    Sums, means and variances are fp32.  a and b are the outputs of sublayers that
+    read the same normed input (a parallel block); c is an addend that enters
+    with unit RMS and a learned per-column weight."""
+    T, W = X.shape
+    if X.dtype != torch.float32 or not X.is_contiguous():
+        raise TypeError("the residual must be contiguous float32")
+    if norm not in NORMS or (norm and norm_w is None) or (norm == "layer" and norm_b is None) or \
+            (c is not None and c_w is None):
+        raise ValueError("residual_step: bad norm / weights")
+    for t, n in ((c_w, "c_w"), (norm_w, "norm_w"), (norm_b, "norm_b")):
+        _fp32_param(t, n)
+    for t in (a, b, c):
+        if t is not None and (t.shape != X.shape or t.stride(-1) != 1 or t.dtype != out_dtype):
+            raise TypeError("residual_step: addends [T, W] with contiguous rows, of the activation dtype")
+    if not X.is_cuda:
+        for t in (a, b):
+            if t is not None:
+                X += t.float()
+        if c is not None:
+            cf = c.float()
+            X += cf * torch.rsqrt((cf * cf).mean(-1, keepdim=True) + eps) * c_w
+        h = None
+        if norm == "rms":
+            h = (X * torch.rsqrt((X * X).mean(-1, keepdim=True) + eps) * norm_w).to(out_dtype)
+        elif norm == "layer":
+            mu = X.mean(-1, keepdim=True)
+            var = ((X - mu) ** 2).mean(-1, keepdim=True)
+            h = ((X - mu) * torch.rsqrt(var + eps) * norm_w + norm_b).to(out_dtype)
+        return h, (X.to(out_dtype) if want_cast else None)
+    h = torch.empty((T, W), dtype=out_dtype, device=X.device) if norm else None
+    xc = torch.empty((T, W), dtype=out_dtype, device=X.device) if want_cast else None
+    _m().residual_step(X.data_ptr(), _ptr(a), a.stride(0) if a is not None else 0, _ptr(b),
+                       b.stride(0) if b is not None else 0, _ptr(c), c.stride(0) if c is not None else 0, _ptr(c_w),
+                       float(eps), NORMS[norm], _ptr(norm_w), _ptr(norm_b), _ptr(h), _ptr(xc), T, W,
+                       int(out_dtype == torch.float32), _stream())
+    return h, xc
 
 
 def stream_step(X: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, gain: torch.Tensor | None,
@@ -111,6 +183,10 @@ def _act(z: torch.Tensor, act: str) -> torch.Tensor:
         return torch.relu(z)
     if act == "silu":
         return z * torch.sigmoid(z)
+    if act == "sigmoid":
+        return torch.sigmoid(z)
+    if act == "relu2":
+        return torch.relu(z) ** 2
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
@@ -123,8 +199,25 @@ def glu_act(gu: torch.Tensor, act: str = "relu") -> torch.Tensor:
     if not gu.is_cuda:
         g, u = gu.float().split(F, dim=1)
         return (_act(g, act) * u).to(gu.dtype)
-    out = torch.empty((T, F), dtype=gu.dtype, device=gu.device)
-    _m().glu_act(out.data_ptr(), gu.data_ptr(), T, F, gu.stride(0), F, ACTS[act], _f32(gu), _stream())
+    return act_mul(gu[:, :F], gu[:, F:], act)
+
+
+def act_mul(gate: torch.Tensor, up: torch.Tensor | None = None, act: str = "silu") -> torch.Tensor:
+    """act(gate) * up, [T, F] (up None: the activation alone).  gate and up may
+    be column sections of wider tensors (contiguous rows, any row stride), e.g.
+    a gate that is part of a fused projection's output."""
+    T, F = gate.shape
+    if act not in ACTS:
+        raise ValueError(f"unknown activation {act!r}")
+    if gate.stride(1) != 1 or (up is not None and (up.shape != gate.shape or up.stride(1) != 1 or
+                                                   up.dtype != gate.dtype)):
+        raise ValueError("act_mul: [T, F] sections with contiguous rows and one dtype")
+    if not gate.is_cuda:
+        o = _act(gate.float(), act)
+        return (o * up.float() if up is not None else o).to(gate.dtype)
+    out = torch.empty((T, F), dtype=gate.dtype, device=gate.device)
+    _m().act_mul(out.data_ptr(), gate.data_ptr(), gate.stride(0), _ptr(up), up.stride(0) if up is not None else 0, T, F,
+                 F, ACTS[act], _f32(gate), _stream())
     return out
 
 
@@ -132,13 +225,16 @@ def glu_act(gu: torch.Tensor, act: str = "relu") -> torch.Tensor:
 def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor, n_q: int, n_k: int, d: int,
                    k_off: int, q_w: torch.Tensor | None, k_w: torch.Tensor | None, eps: float,
                    temp: tuple[float, float] | None, kc: torch.Tensor, vc: torch.Tensor | None, v_mode: int = 0,
-                   v_off: int = 0, v_w: int = 0) -> None:
+                   v_off: int = 0, v_w: int = 0, v_first: torch.Tensor | None = None, v_lambda: float = 0.0) -> None:
     """Per row of the fused projection output x = [q | k | v] (in place):
     q heads: unit RMS times q_w (when given) and the position gain
     1 + coef * ln(floor((p + 1) / every) + 1) (temp = (coef, every));
     k heads at column k_off: unit RMS times k_w (when given) into the K cache;
     v_mode 0: no V cache; 1: the k columns as projected are the value;
-    2: the v_w columns at v_off are.  Rows with slot < 0 cache nothing."""
+    2: the v_w columns at v_off are.  With v_first [T, v_w] (v_mode 2; the same
+    tokens' values of an earlier layer, a column section of any row stride) the
+    cached value is (1 - v_lambda) v + v_lambda v_first, formed in fp32.
+    Rows with slot < 0 cache nothing."""
     T = x.shape[0]
     coef, every = (float(temp[0]), float(temp[1])) if temp else (0.0, 1.0)
     _fp32_param(q_w, "q_w")
@@ -150,6 +246,9 @@ def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor
         raise ValueError("headprep_cache: cache row widths do not match the sections")
     if max(n_q * d, k_off + k_wd, (v_off + v_w) if v_mode == 2 else 0) > x.shape[1]:
         raise ValueError("headprep_cache: sections exceed the row")
+    if v_first is not None and (v_mode != 2 or v_first.shape != (T, v_w) or v_first.stride(1) != 1 or
+                                v_first.dtype != x.dtype):
+        raise ValueError("headprep_cache: v_first is [T, v_w] of x's dtype, with v_mode 2")
     if not x.is_cuda:
         xf = x.float()
         if q_w is not None or coef != 0.0:
@@ -170,13 +269,17 @@ def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor
             k = (kh * torch.rsqrt((kh * kh).mean(-1, keepdim=True) + eps) * k_w).reshape(-1, k_wd)
         kc[sl] = k.to(kc.dtype)
         if v_mode == 2:
-            vc[sl] = x[ok, v_off:v_off + v_w]
+            v = x[ok, v_off:v_off + v_w]
+            if v_first is not None:
+                v = ((1.0 - v_lambda) * v.float() + v_lambda * v_first[ok].float()).to(x.dtype)
+            vc[sl] = v
         return
     if positions.dtype != torch.int64 or slots.dtype != torch.int64:
         raise TypeError("positions and slots must be int64")
     _m().headprep_cache(x.data_ptr(), x.stride(0), positions.data_ptr(), slots.data_ptr(), T, n_q, n_k, d, k_off,
                         _ptr(q_w), _ptr(k_w), float(eps), coef, every, kc.data_ptr(), _ptr(vc) if v_mode else 0,
-                        v_mode, v_off, v_w, _f32(x), _stream())
+                        v_mode, v_off, v_w, _ptr(v_first), v_first.stride(0) if v_first is not None else 0,
+                        float(v_lambda), _f32(x), _stream())
 
 
 # ----------------------------------------------------------------- attention
@@ -215,7 +318,8 @@ def tile_attention_ok(q: torch.Tensor, d: int, dv: int) -> bool:
 def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
               seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
               group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
-              out_f32: bool = False, tiles: torch.Tensor | None = None, n_tile_rows: int = 0) -> torch.Tensor:
+              out_f32: bool = False, tiles: torch.Tensor | None = None, n_tile_rows: int = 0, softcap: float = 0.0,
+              dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
     """Attention of one step's rows: the first n_tile_rows rows (prompt chunks,
     cut into `tiles` [n, 2] = first row, row count) on the matrix-core prefill
     kernel where it applies, all other rows (decode tokens; every row when it
@@ -224,7 +328,8 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     T = q.shape[0]
     if not tile_attention_ok(q, d, dv) or not scale > 0:  # the matrix-core kernels fold a positive scale
         return row_attention(q, kc, vc, positions, seq, block_tables, block_size, n_qh, maps, group, d, dv, scale,
-                             mask, size, parts, out_f32)
+                             mask, size, parts, out_f32, softcap, dist_bias)
+    _check_score_terms(softcap, dist_bias, n_qh)
     if tiles is None:
         n_tile_rows = 0
     if kc.dtype != q.dtype or vc.dtype != q.dtype or not kc.is_contiguous() or not vc.is_contiguous() or \
@@ -240,7 +345,8 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     odt = torch.float32 if out_f32 else q.dtype
     out = torch.empty((T, n_qh, dv), dtype=odt, device=q.device)
     common = (block_tables.data_ptr(), block_tables.stride(0), block_size)
-    heads = (n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale), MASKS[mask], int(size))
+    heads = (n_qh, maps, group, d, dv, kc.shape[-1], vc.shape[-1], float(scale), MASKS[mask], int(size),
+             float(softcap), _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0)
     if n_tile_rows:
         if seq is None or tiles.dtype != torch.int32 or not tiles.is_contiguous():
             raise TypeError("attention: prompt-chunk rows need seq and int32 tiles")
@@ -257,15 +363,30 @@ def attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: to
     return out
 
 
+def _check_score_terms(softcap: float, dist_bias, n_qh: int) -> None:
+    if softcap < 0:
+        raise ValueError("softcap must be positive (0: none)")
+    if dist_bias is not None:
+        for t in dist_bias:
+            _fp32_param(t, "dist_bias")
+            if t.numel() != n_qh:
+                raise ValueError("dist_bias: one (r1, r2) pair per query vector")
+
+
 def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions: torch.Tensor,
                   seq: torch.Tensor | None, block_tables: torch.Tensor, block_size: int, n_qh: int, maps: int,
                   group: int, d: int, dv: int, scale: float, mask: str = "causal", size: int = 0, parts: int = 1,
-                  out_f32: bool = False) -> torch.Tensor:
+                  out_f32: bool = False, softcap: float = 0.0,
+                  dist_bias: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
     """Softmax attention of T rows over their sequences' paged caches.
     q [T, >= n_qh * d] (n_qh = heads * maps query vectors per row); returns
     [T, n_qh, dv].  Query vector qh reads K head (qh // maps // group) * maps +
-    qh % maps and V head qh // maps // group."""
+    qh % maps and V head qh // maps // group.  The score of query position i
+    and key position j is s = q . k * scale; with softcap > 0 then
+    s <- softcap * tanh(s / softcap); with dist_bias = (r1, r2), fp32 [n_qh]
+    each, then s <- s - r1[qh] * ln(1 + r2[qh] * (i - j))."""
     T = q.shape[0]
+    _check_score_terms(softcap, dist_bias, n_qh)
     if mask not in MASKS:
         raise ValueError(f"unknown mask {mask!r}")
     if mask != "causal" and size < 1:
@@ -293,6 +414,11 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
             K = kc[sl].float()[:, : n_kh * d].reshape(n, n_kh, d)[:, kh]  # [n, n_qh, d]
             V = vc[sl].float()[:, : (n_qh // maps // group) * dv].reshape(n, -1, dv)[:, vh]
             sc = torch.einsum("ihd,jhd->hij", qf[rows], K) * scale
+            if softcap:
+                sc = softcap * torch.tanh(sc / softcap)
+            if dist_bias is not None:
+                dist = (p[:, None] - j[None, :]).clamp_min(0).float()
+                sc = sc - dist_bias[0][:, None, None] * torch.log1p(dist_bias[1][:, None, None] * dist[None])
             vis = (j[None, :] <= p[:, None]) & (j[None, :] >= first_visible(p, mask, size)[:, None])
             sc = sc.masked_fill(~vis[None], float("-inf"))
             out[rows] = torch.einsum("hij,jhd->ihd", torch.softmax(sc, -1), V)
@@ -308,7 +434,8 @@ def row_attention(q: torch.Tensor, kc: torch.Tensor, vc: torch.Tensor, positions
     ws = torch.empty((T, n_qh, parts, 2 + dv), dtype=torch.float32, device=q.device) if parts > 1 else None
     _m().row_attention(out.data_ptr(), _ptr(ws), q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(),
                        positions.data_ptr(), _ptr(seq), block_tables.data_ptr(), block_tables.stride(0), block_size,
-                       T, n_qh, maps, group, d, dv, Wk, Wv, float(scale), MASKS[mask], int(size), parts, _f32(q),
+                       T, n_qh, maps, group, d, dv, Wk, Wv, float(scale), MASKS[mask], int(size), float(softcap),
+                       _ptr(dist_bias[0]) if dist_bias else 0, _ptr(dist_bias[1]) if dist_bias else 0, parts, _f32(q),
                        int(odt == torch.float32), _stream())
     return out
 
