@@ -16,19 +16,31 @@ using u = uintptr_t;
 extern "C" {
 int dxm_stream_step(float*, const void*, int64_t, const float*, const float*, const float*, const float*, float, void*,
                     int64_t, int, int, int, int, hipStream_t);
-int dxm_embed_streams(float*, const void*, const int64_t*, int, int, int, int64_t, int, hipStream_t);
-int dxm_glu_act(void*, const void*, int, int, int64_t, int64_t, int, int, hipStream_t);
+int dxm_embed_streams(float*, const void*, const int64_t*, int, int, int, int64_t, const void*, const int64_t*,
+                      int64_t, int, hipStream_t);
+int dxm_gather_rows(void*, const void*, const int64_t*, int, int, int64_t, int, hipStream_t);
+int dxm_residual_step(float*, const void*, int64_t, const void*, int64_t, const void*, int64_t, const float*, float,
+                      int, const float*, const float*, void*, void*, int, int, int, hipStream_t);
+int dxm_act_mul(void*, const void*, int64_t, const void*, int64_t, int, int, int64_t, int, int, hipStream_t);
 int dxm_headprep_cache(void*, int64_t, const int64_t*, const int64_t*, int, int, int, int, int, const float*,
-                       const float*, float, float, double, void*, void*, int, int, int, int, hipStream_t);
+                       const float*, float, float, double, void*, void*, int, int, int, const void*, int64_t, float,
+                       int, hipStream_t);
+int dxm_moe_route(int*, float*, const float*, const float*, int, int, int, int, int, hipStream_t);
+int dxm_moe_plan(int*, int*, const int*, int, int, hipStream_t);
+int dxm_grouped_gemm(void*, const void*, int64_t, const void*, const int*, const int*, int, int, int, int, int, int,
+                     int, int, hipStream_t);
+int dxm_moe_combine(void*, const void*, const float*, const void*, int64_t, int, int, int, int, hipStream_t);
 int dxm_diff_combine(void*, const float*, int64_t, int, float, float, float, int, hipStream_t);
 int dxm_row_attention(void*, float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*,
-                      const int*, int, int, int, int, int, int, int, int, int, int, float, int, int, int, int, int,
-                      hipStream_t);
+                      const int*, int, int, int, int, int, int, int, int, int, int, float, int, int, float, const float*,
+                      const float*, int, int, int, hipStream_t);
 int dxm_tile_attention_ok(int, int);
 int dxm_tile_attention(void*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*,
-                       int, int, const int*, int, int, int, int, int, int, int, int, float, int, int, int, hipStream_t);
+                       int, int, const int*, int, int, int, int, int, int, int, int, float, int, int, float, const float*,
+                       const float*, int, hipStream_t);
 int dxm_group_decode(float*, const void*, int64_t, const void*, const void*, const int64_t*, const int*, const int*, int,
-                     int, int, int, int, int, int, int, int, int, float, int, int, int, hipStream_t);
+                     int, int, int, int, int, int, int, int, int, float, int, int, float, const float*, const float*, int,
+                     hipStream_t);
 int dxm_merge_parts(void*, const float*, int64_t, int, int, int, hipStream_t);
 }
 
@@ -48,19 +60,50 @@ PYBIND11_MODULE(_C_mixers, m) {
     check(dxm_stream_step(F(X), P(y), ys, F(mix), F(gain), F(rin), F(nw), eps, P(out), os, rows, S_, W, f32, S(st)),
           "stream_step");
   });
-  m.def("embed_streams", [](u X, u table, u ids, int rows, int S_, int W, int64_t vocab, int f32, u st) {
-    check(dxm_embed_streams(F(X), P(table), reinterpret_cast<const int64_t*>(ids), rows, S_, W, vocab, f32, S(st)),
+  m.def("embed_streams", [](u X, u table, u ids, int rows, int S_, int W, int64_t vocab, u ptab, u pos, int64_t n_pos,
+                            int f32, u st) {
+    check(dxm_embed_streams(F(X), P(table), reinterpret_cast<const int64_t*>(ids), rows, S_, W, vocab, P(ptab),
+                            reinterpret_cast<const int64_t*>(pos), n_pos, f32, S(st)),
           "embed_streams");
   });
-  m.def("glu_act", [](u out, u gu, int rows, int Fw, int64_t is, int64_t os, int act, int f32, u st) {
-    check(dxm_glu_act(P(out), P(gu), rows, Fw, is, os, act, f32, S(st)), "glu_act");
+  m.def("gather_rows", [](u out, u table, u ids, int rows, int W, int64_t vocab, int f32, u st) {
+    check(dxm_gather_rows(P(out), P(table), reinterpret_cast<const int64_t*>(ids), rows, W, vocab, f32, S(st)),
+          "gather_rows");
+  });
+  m.def("residual_step", [](u X, u a, int64_t as, u b, int64_t bs, u c, int64_t cs, u cw, float eps, int norm, u nw,
+                            u nb, u out, u xc, int rows, int W, int f32, u st) {
+    check(dxm_residual_step(F(X), P(a), as, P(b), bs, P(c), cs, F(cw), eps, norm, F(nw), F(nb), P(out), P(xc), rows, W,
+                            f32, S(st)),
+          "residual_step");
+  });
+  m.def("act_mul", [](u out, u gate, int64_t gs, u up, int64_t us, int rows, int Fw, int64_t os, int act, int f32,
+                      u st) {
+    check(dxm_act_mul(P(out), P(gate), gs, P(up), us, rows, Fw, os, act, f32, S(st)), "act_mul");
+  });
+  m.def("moe_route", [](u idx, u w, u z, u corr, int T, int E, int top, int n_groups, int keep, u st) {
+    check(dxm_moe_route(reinterpret_cast<int*>(idx), F(w), F(z), F(corr), T, E, top, n_groups, keep, S(st)),
+          "moe_route");
+  });
+  m.def("moe_plan", [](u order, u offsets, u idx, int R, int E, u st) {
+    check(dxm_moe_plan(reinterpret_cast<int*>(order), reinterpret_cast<int*>(offsets),
+                       reinterpret_cast<const int*>(idx), R, E, S(st)),
+          "moe_plan");
+  });
+  m.def("grouped_gemm", [](u out, u a, int64_t as, u w, u order, u offsets, int R, int E, int N, int K, int top,
+                           int gather, int scatter, int f32, u st) {
+    check(dxm_grouped_gemm(P(out), P(a), as, P(w), reinterpret_cast<const int*>(order),
+                           reinterpret_cast<const int*>(offsets), R, E, N, K, top, gather, scatter, f32, S(st)),
+          "grouped_gemm");
+  });
+  m.def("moe_combine", [](u out, u y, u w, u shared, int64_t ss, int T, int top, int W, int f32, u st) {
+    check(dxm_moe_combine(P(out), P(y), F(w), P(shared), ss, T, top, W, f32, S(st)), "moe_combine");
   });
   m.def("headprep_cache", [](u x, int64_t xs, u pos, u slots, int rows, int n_q, int n_k, int d, int k_off, u qw, u kw,
-                             float eps, float coef, double every, u kc, u vc, int v_mode, int v_off, int v_w, int f32,
-                             u st) {
+                             float eps, float coef, double every, u kc, u vc, int v_mode, int v_off, int v_w, u vf,
+                             int64_t vfs, float lam, int f32, u st) {
     check(dxm_headprep_cache(P(x), xs, reinterpret_cast<const int64_t*>(pos), reinterpret_cast<const int64_t*>(slots),
                              rows, n_q, n_k, d, k_off, F(qw), F(kw), eps, coef, every, P(kc), P(vc), v_mode, v_off,
-                             v_w, f32, S(st)),
+                             v_w, P(vf), vfs, lam, f32, S(st)),
           "headprep_cache");
   });
   m.def("diff_combine", [](u out, u a, int64_t n_vec, int dv, float lam, float post, float eps, int f32, u st) {
@@ -69,28 +112,29 @@ PYBIND11_MODULE(_C_mixers, m) {
   m.def("tile_attention_ok", &dxm_tile_attention_ok);
   m.def("tile_attention", [](u out, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, u tiles,
                              int n_tiles, int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale,
-                             int mask, int size, int out_f32, u st) {
+                             int mask, int size, float cap, u r1, u r2, int out_f32, u st) {
     check(dxm_tile_attention(P(out), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                              reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs,
                              reinterpret_cast<const int*>(tiles), n_tiles, n_qh, maps, group, d, dv, Wk, Wv, scale,
-                             mask, size, out_f32, S(st)),
+                             mask, size, cap, F(r1), F(r2), out_f32, S(st)),
           "tile_attention");
   });
   m.def("group_decode", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                            int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                           int size, int parts, int out_f32, u st) {
+                           int size, float cap, u r1, u r2, int parts, int out_f32, u st) {
     check(dxm_group_decode(F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                            reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
-                           maps, group, d, dv, Wk, Wv, scale, mask, size, parts, S(st)),
+                           maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), parts, S(st)),
           "group_decode");
     check(dxm_merge_parts(P(out), F(ws), (int64_t)rows * n_qh, parts, dv, out_f32, S(st)), "merge_parts");
   });
   m.def("row_attention", [](u out, u ws, u q, int64_t qs, u kc, u vc, u pos, u seq, u bt, int bts, int bs, int rows,
                             int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                            int size, int parts, int f32, int out_f32, u st) {
+                            int size, float cap, u r1, u r2, int parts, int f32, int out_f32, u st) {
     check(dxm_row_attention(P(out), F(ws), P(q), qs, P(kc), P(vc), reinterpret_cast<const int64_t*>(pos),
                             reinterpret_cast<const int*>(seq), reinterpret_cast<const int*>(bt), bts, bs, rows, n_qh,
-                            maps, group, d, dv, Wk, Wv, scale, mask, size, parts, f32, out_f32, S(st)),
+                            maps, group, d, dv, Wk, Wv, scale, mask, size, cap, F(r1), F(r2), parts, f32, out_f32,
+                            S(st)),
           "row_attention");
   });
 }

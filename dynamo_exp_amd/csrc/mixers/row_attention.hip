@@ -7,7 +7,10 @@
 //     causal:  0 .. p          window: max(0, p - size + 1) .. p
 //     chunk:   floor(p / size) * size .. p
 // counted in sequence positions, so the result does not depend on how a prompt
-// was cut into steps.  Scores, softmax weights and the weighted sum are fp32;
+// was cut into steps.  The score of query position p and key position j is
+// s = q . k * scale, optionally capped, s <- cap * tanh(s / cap), and optionally
+// lowered by a per-head penalty that grows with the logarithm of the distance,
+// s <- s - r1[qh] * ln(1 + r2[qh] * (p - j)).  Scores, softmax weights and the weighted sum are fp32;
 // q, the caches and the output are bf16 or fp32 (the output optionally fp32
 // beside bf16 caches).
 //
@@ -67,6 +70,9 @@ struct RowAttnArgs {
   int mask;  // 0 causal, 1 window, 2 chunk
   int size;
   int parts;
+  float softcap;    // 0: scores are not capped
+  const float* r1;  // [n_qh] distance penalty (null: none)
+  const float* r2;
 };
 
 template <typename T, typename OutT, int NV>
@@ -92,6 +98,8 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
   const int64_t tpp = (tiles + a.parts - 1) / a.parts;
   const int64_t t0 = part * tpp, t1 = t0 + tpp < tiles ? t0 + tpp : tiles;
   const bool vec = a.d % Elem<T>::kVec == 0 && a.Wk % Elem<T>::kVec == 0;
+  const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  const float r1 = a.r1 ? a.r1[qh] : 0.f, r2 = a.r1 ? a.r2[qh] : 0.f;
   float mx = -INFINITY, l = 0.f;
   float acc[NV];
 #pragma unroll
@@ -110,6 +118,8 @@ __global__ void __launch_bounds__(64) row_attention_kernel(RowAttnArgs a) {
       } else {
         for (int e = 0; e < a.d; ++e) sum += Elem<T>::ld(k, e) * qs[e];
       }
+      if (cap > 0.f) sum = cap * tanhf(sum * inv_cap);
+      if (a.r1) sum -= r1 * log1pf(r2 * (float)(p - j));
       s = sum;
     }
     const float mn = fmaxf(mx, wave_reduce_max(s));
@@ -211,14 +221,16 @@ int launch_rows(const RowAttnArgs& a, int rows, hipStream_t st) {
 extern "C" int dxm_row_attention(void* out, float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc,
                                  const int64_t* pos, const int* seq, const int* bt, int bt_stride, int bs, int rows,
                                  int n_qh, int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask,
-                                 int size, int parts, int f32, int out_f32, hipStream_t st) {
+                                 int size, float softcap, const float* r1, const float* r2, int parts, int f32,
+                                 int out_f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group) return 1;
   if (d < 1 || dv < 1 || dv > 1024 || d > 8192) return 2;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535 || n_qh > 65535) return 3;
   if (parts > 1 && !ws) return 4;
+  if (softcap < 0.f || (r1 && !r2)) return 6;
   RowAttnArgs a{q, q_stride, kc, vc, out, ws, pos, seq, bt, bt_stride, bs, n_qh, maps, group,
-                d, dv, Wk, Wv, scale, mask, size, parts};
+                d, dv, Wk, Wv, scale, mask, size, parts, softcap, r1, r2};
   if (f32) return launch_rows<float, float>(a, rows, st);
   if (out_f32) return launch_rows<bf16_t, float>(a, rows, st);
   return launch_rows<bf16_t, bf16_t>(a, rows, st);

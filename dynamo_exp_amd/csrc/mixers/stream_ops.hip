@@ -2,7 +2,9 @@
 // residual ("hyper-connections") update fused with the next sublayer's
 // read-in and RMS norm, the embedding gather into fp32 streams, gated
 // feed-forward activations, per-head q/k normalisation fused with the paged
-// cache write, and the two-map (differential) attention combine.
+// cache write, the two-map (differential) attention combine, and the
+// single-residual step of parallel blocks (several sublayer outputs and a
+// unit-RMS addend joined in one pass with the next RMS or layer norm).
 //
 // Every kernel is a template over the activation element (bf16 bits or
 // float); reductions, norms, the residual streams and every scale are fp32
@@ -144,38 +146,198 @@ __global__ void __launch_bounds__(kThreads) stream_step_kernel(float* __restrict
   }
 }
 
-// X[t, s, :] = table[ids[t], :] for every stream s (fp32 streams)
+// X[t, s, :] = table[ids[t], :] (+ ptab[pos[t], :], a learned vector per position)
+// for every stream s (fp32 streams; the sum is fp32)
 template <typename T>
 __global__ void __launch_bounds__(kThreads) embed_streams_kernel(float* __restrict__ X, const T* __restrict__ table,
                                                                  const int64_t* __restrict__ ids, int S, int W,
-                                                                 int64_t vocab) {
+                                                                 int64_t vocab, const T* __restrict__ ptab,
+                                                                 const int64_t* __restrict__ pos, int64_t n_pos) {
   const int64_t t = blockIdx.x;
   const int64_t id = ids[t];
   const bool ok = id >= 0 && id < vocab;
+  const int64_t p = ptab ? pos[t] : -1;
+  const bool pok = p >= 0 && p < n_pos;
   for (int c = threadIdx.x; c < W; c += kThreads) {
-    const float v = ok ? ldf<T>(table, id * (int64_t)W + c) : 0.f;
+    float v = ok ? ldf<T>(table, id * (int64_t)W + c) : 0.f;
+    if (pok) v += ldf<T>(ptab, p * (int64_t)W + c);
     for (int s = 0; s < S; ++s) X[(t * S + s) * (int64_t)W + c] = v;
+  }
+}
+
+// out[t, :] = table[ids[t], :] (zeros for ids outside the table)
+template <typename T>
+__global__ void __launch_bounds__(kThreads) gather_rows_kernel(T* __restrict__ out, const T* __restrict__ table,
+                                                               const int64_t* __restrict__ ids, int W, int64_t vocab) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = ids[t];
+  const bool ok = id >= 0 && id < vocab;
+  for (int c = threadIdx.x; c < W; c += kThreads) out[t * (int64_t)W + c] = ok ? table[id * (int64_t)W + c] : (T)0;
+}
+
+// One step of a single fp32 residual x [rows, W], in place:
+//     x <- x + a + b + c / sqrt(mean(c^2) + eps) * cw        (a, b, c optional)
+// then  xc = x in T (when xc), and the norm that follows (when out):
+//     norm 1 (RMS):    out = x / sqrt(mean(x^2) + eps) * nw
+//     norm 2 (layer):  out = (x - mean) / sqrt(mean((x - mean)^2) + eps) * nw + nb
+// The row stays in registers between the passes (W <= kThreads * V * kResChunks)
+// or is re-read from x by the thread that wrote it.
+constexpr int kResChunks = 8;
+template <typename T, int V>
+__global__ void __launch_bounds__(kThreads) residual_step_kernel(
+    float* __restrict__ X, const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
+    const T* __restrict__ c, int64_t c_stride, const float* __restrict__ cw, float eps, int norm,
+    const float* __restrict__ nw, const float* __restrict__ nb, T* __restrict__ out, T* __restrict__ xc, int W) {
+  __shared__ float red[16];
+  const int64_t row = blockIdx.x;
+  float* x = X + row * (int64_t)W;
+  float rc = 0.f;
+  if (c) {
+    float ss = 0.f;
+    for (int e = threadIdx.x * V; e < W; e += kThreads * V) {
+      float v[V];
+      ldv<T, V>(c + row * c_stride + e, v);
+#pragma unroll
+      for (int i = 0; i < V; ++i) ss += v[i] * v[i];
+    }
+    rc = rsqrtf(block_reduce_sum(ss, red) / (float)W + eps);
+    __syncthreads();
+  }
+  const bool keep = W <= kThreads * V * kResChunks;
+  float r[kResChunks][V];
+  float sum = 0.f;
+  const bool touch = a || b || c;
+#pragma unroll
+  for (int k = 0; k < kResChunks; ++k) {
+    const int e = (threadIdx.x + k * kThreads) * V;
+    if (e < W) {
+      ldv<float, V>(x + e, r[k]);
+      float t[V];
+      if (a) {
+        ldv<T, V>(a + row * a_stride + e, t);
+#pragma unroll
+        for (int i = 0; i < V; ++i) r[k][i] += t[i];
+      }
+      if (b) {
+        ldv<T, V>(b + row * b_stride + e, t);
+#pragma unroll
+        for (int i = 0; i < V; ++i) r[k][i] += t[i];
+      }
+      if (c) {
+        float w[V];
+        ldv<T, V>(c + row * c_stride + e, t);
+        ldv<float, V>(cw + e, w);
+#pragma unroll
+        for (int i = 0; i < V; ++i) r[k][i] += t[i] * rc * w[i];
+      }
+      if (touch) stv<float, V>(x + e, r[k]);
+      if (xc) stv<T, V>(xc + row * (int64_t)W + e, r[k]);
+#pragma unroll
+      for (int i = 0; i < V; ++i) sum += r[k][i];
+    }
+  }
+  if (!keep) {  // wide rows: the same arithmetic, chunk by chunk through x
+    for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
+      float v[V], t[V];
+      ldv<float, V>(x + e, v);
+      if (a) {
+        ldv<T, V>(a + row * a_stride + e, t);
+#pragma unroll
+        for (int i = 0; i < V; ++i) v[i] += t[i];
+      }
+      if (b) {
+        ldv<T, V>(b + row * b_stride + e, t);
+#pragma unroll
+        for (int i = 0; i < V; ++i) v[i] += t[i];
+      }
+      if (c) {
+        float w[V];
+        ldv<T, V>(c + row * c_stride + e, t);
+        ldv<float, V>(cw + e, w);
+#pragma unroll
+        for (int i = 0; i < V; ++i) v[i] += t[i] * rc * w[i];
+      }
+      if (touch) stv<float, V>(x + e, v);
+      if (xc) stv<T, V>(xc + row * (int64_t)W + e, v);
+#pragma unroll
+      for (int i = 0; i < V; ++i) sum += v[i];
+    }
+  }
+  if (!norm) return;
+  float mean = 0.f;
+  if (norm == 2) {
+    mean = block_reduce_sum(sum, red) / (float)W;
+    __syncthreads();
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < kResChunks; ++k) {
+    const int e = (threadIdx.x + k * kThreads) * V;
+    if (e < W) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) ss += (r[k][i] - mean) * (r[k][i] - mean);
+    }
+  }
+  if (!keep) {
+    for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
+      float v[V];
+      ldv<float, V>(x + e, v);
+#pragma unroll
+      for (int i = 0; i < V; ++i) ss += (v[i] - mean) * (v[i] - mean);
+    }
+  }
+  const float rs = rsqrtf(block_reduce_sum(ss, red) / (float)W + eps);
+#pragma unroll
+  for (int k = 0; k < kResChunks; ++k) {
+    const int e = (threadIdx.x + k * kThreads) * V;
+    if (e < W) {
+      float w[V], bb[V], o[V];
+      ldv<float, V>(nw + e, w);
+      if (norm == 2) ldv<float, V>(nb + e, bb);
+#pragma unroll
+      for (int i = 0; i < V; ++i) o[i] = (r[k][i] - mean) * rs * w[i] + (norm == 2 ? bb[i] : 0.f);
+      stv<T, V>(out + row * (int64_t)W + e, o);
+    }
+  }
+  if (!keep) {
+    for (int e = (threadIdx.x + kResChunks * kThreads) * V; e < W; e += kThreads * V) {
+      float v[V], w[V], bb[V], o[V];
+      ldv<float, V>(x + e, v);
+      ldv<float, V>(nw + e, w);
+      if (norm == 2) ldv<float, V>(nb + e, bb);
+#pragma unroll
+      for (int i = 0; i < V; ++i) o[i] = (v[i] - mean) * rs * w[i] + (norm == 2 ? bb[i] : 0.f);
+      stv<T, V>(out + row * (int64_t)W + e, o);
+    }
   }
 }
 
 __device__ __forceinline__ float act_fn(float z, int act) {
   if (act == 0) return fmaxf(z, 0.f);           // relu
   if (act == 1) return z / (1.f + __expf(-z));  // silu
+  if (act == 3) return 1.f / (1.f + __expf(-z));  // sigmoid
+  if (act == 4) {                                 // relu squared
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+  }
   const float c = 0.7978845608028654f;          // gelu, tanh form
   return 0.5f * z * (1.f + tanhf(c * (z + 0.044715f * z * z * z)));
 }
 
-// gu [rows, 2F] = [gate | up]  ->  out [rows, F] = act(gate) * up
+// out [rows, F] = act(gate) * up  (up null: act(gate)); gate and up are column
+// sections of wider rows (a gated feed-forward's [gate | up], an output gate
+// that is part of a fused projection)
 template <typename T, int V>
-__global__ void __launch_bounds__(kThreads) glu_act_kernel(T* __restrict__ out, const T* __restrict__ gu, int F,
-                                                           int64_t in_stride, int64_t out_stride, int act) {
+__global__ void __launch_bounds__(kThreads) act_mul_kernel(T* __restrict__ out, const T* __restrict__ gate,
+                                                           int64_t g_stride, const T* __restrict__ up,
+                                                           int64_t u_stride, int F, int64_t out_stride, int act) {
   const int64_t r = blockIdx.y;
   for (int c = (blockIdx.x * kThreads + threadIdx.x) * V; c < F; c += gridDim.x * kThreads * V) {
     float g[V], u[V], o[V];
-    ldv<T, V>(gu + r * in_stride + c, g);
-    ldv<T, V>(gu + r * in_stride + F + c, u);
+    ldv<T, V>(gate + r * g_stride + c, g);
+    if (up) ldv<T, V>(up + r * u_stride + c, u);
 #pragma unroll
-    for (int e = 0; e < V; ++e) o[e] = act_fn(g[e], act) * u[e];
+    for (int e = 0; e < V; ++e) o[e] = act_fn(g[e], act) * (up ? u[e] : 1.f);
     stv<T, V>(out + r * out_stride + c, o);
   }
 }
@@ -186,14 +348,16 @@ __global__ void __launch_bounds__(kThreads) glu_act_kernel(T* __restrict__ out, 
 //   k: n_k vectors of d at column k_off; with kw: unit RMS times kw; written to
 //      the K cache row of the token's slot (kc [slots, n_k * d])
 //   v: v_mode 0: no V cache (V is the K cache); 1: the k section as projected
-//      (before its norm) is the value; 2: v_w columns at v_off are the value
+//      (before its norm) is the value; 2: v_w columns at v_off are the value,
+//      mixed with an earlier layer's values of the same token when v_first is
+//      given: (1 - v_lambda) v + v_lambda v_first, in fp32
 // slot < 0: nothing is cached for the row.
 template <typename T, int V>
 __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
     T* __restrict__ x, int64_t x_stride, const int64_t* __restrict__ pos, const int64_t* __restrict__ slots,
     int n_q, int n_k, int d, int k_off, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
     float temp_coef, double temp_every, T* __restrict__ kc, T* __restrict__ vc, int v_mode, int v_off, int v_w,
-    int lpv) {
+    const T* __restrict__ v_first, int64_t vf_stride, float v_lambda, int lpv) {
   // lpv lanes (a power of two) share one head vector, so a wave works on 64 / lpv
   // vectors at once and their loads overlap; the sum of squares is reduced inside the group
   const int64_t t = blockIdx.x;
@@ -242,7 +406,19 @@ __global__ void __launch_bounds__(kThreads) headprep_cache_kernel(
   if (v_mode == 2 && slot >= 0) {
     const T* vs = row + v_off;
     T* vd = vc + slot * (int64_t)v_w;
-    for (int e = threadIdx.x * V; e < v_w; e += kThreads * V) cpv<T, V>(vd + e, vs + e);
+    if (v_first) {
+      const T* vf = v_first + t * vf_stride;
+      for (int e = threadIdx.x * V; e < v_w; e += kThreads * V) {
+        float a[V], f[V];
+        ldv<T, V>(vs + e, a);
+        ldv<T, V>(vf + e, f);
+#pragma unroll
+        for (int i = 0; i < V; ++i) a[i] = (1.f - v_lambda) * a[i] + v_lambda * f[i];
+        stv<T, V>(vd + e, a);
+      }
+    } else {
+      for (int e = threadIdx.x * V; e < v_w; e += kThreads * V) cpv<T, V>(vd + e, vs + e);
+    }
   }
 }
 
@@ -301,34 +477,69 @@ int dxm_stream_step(float* X, const void* y, int64_t y_stride, const float* mix,
   return 0;
 }
 
-int dxm_embed_streams(float* X, const void* table, const int64_t* ids, int rows, int S, int W, int64_t vocab, int f32,
-                      hipStream_t st) {
+int dxm_embed_streams(float* X, const void* table, const int64_t* ids, int rows, int S, int W, int64_t vocab,
+                      const void* ptab, const int64_t* pos, int64_t n_pos, int f32, hipStream_t st) {
   if (rows <= 0) return 0;
+  if (ptab && !pos) return 1;
   DISPATCH_T(f32, hipLaunchKernelGGL(embed_streams_kernel<T>, dim3(rows), dim3(kThreads), 0, st, X, (const T*)table,
-                                     ids, S, W, vocab));
+                                     ids, S, W, vocab, (const T*)ptab, pos, n_pos));
   DX_CHECK_LAUNCH();
   return 0;
 }
 
-int dxm_glu_act(void* out, const void* gu, int rows, int F, int64_t in_stride, int64_t out_stride, int act, int f32,
-                hipStream_t st) {
-  if (rows <= 0 || F <= 0) return 0;
-  if (act < 0 || act > 2) return 1;
+int dxm_gather_rows(void* out, const void* table, const int64_t* ids, int rows, int W, int64_t vocab, int f32,
+                    hipStream_t st) {
+  if (rows <= 0) return 0;
+  DISPATCH_T(f32, hipLaunchKernelGGL(gather_rows_kernel<T>, dim3(rows), dim3(kThreads), 0, st, (T*)out,
+                                     (const T*)table, ids, W, vocab));
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_residual_step(float* X, const void* a, int64_t a_stride, const void* b, int64_t b_stride, const void* c,
+                      int64_t c_stride, const float* cw, float eps, int norm, const float* nw, const float* nb,
+                      void* out, void* xc, int rows, int W, int f32, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (W < 1 || norm < 0 || norm > 2) return 1;
+  if ((c && !cw) || (norm && (!nw || !out)) || (norm == 2 && !nb)) return 2;
   const int esz = f32 ? 4 : 2;
-  const bool vec = F % 4 == 0 && in_stride % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)gu % (4 * esz) == 0 &&
+  auto al = [&](const void* p, int by) { return (uintptr_t)p % by == 0; };
+  const bool vec = W % 4 == 0 && a_stride % 4 == 0 && b_stride % 4 == 0 && c_stride % 4 == 0 && al(X, 16) &&
+                   al(a, 4 * esz) && al(b, 4 * esz) && al(c, 4 * esz) && al(cw, 16) && al(nw, 16) && al(nb, 16) &&
+                   al(out, 4 * esz) && al(xc, 4 * esz);
+  if (vec) {
+    DISPATCH_T(f32, hipLaunchKernelGGL((residual_step_kernel<T, 4>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)a,
+                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, eps, norm, nw, nb,
+                                       (T*)out, (T*)xc, W));
+  } else {
+    DISPATCH_T(f32, hipLaunchKernelGGL((residual_step_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, st, X, (const T*)a,
+                                       a_stride, (const T*)b, b_stride, (const T*)c, c_stride, cw, eps, norm, nw, nb,
+                                       (T*)out, (T*)xc, W));
+  }
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+int dxm_act_mul(void* out, const void* gate, int64_t g_stride, const void* up, int64_t u_stride, int rows, int F,
+                int64_t out_stride, int act, int f32, hipStream_t st) {
+  if (rows <= 0 || F <= 0) return 0;
+  if (act < 0 || act > 4) return 1;
+  const int esz = f32 ? 4 : 2;
+  const bool vec = F % 4 == 0 && g_stride % 4 == 0 && u_stride % 4 == 0 && out_stride % 4 == 0 &&
+                   (uintptr_t)gate % (4 * esz) == 0 && (uintptr_t)up % (4 * esz) == 0 &&
                    (uintptr_t)out % (4 * esz) == 0;
   const int per = kThreads * (vec ? 4 : 1);
   const int gx = (F + per - 1) / per;
   for (int r0 = 0; r0 < rows; r0 += 65535) {
     const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
     if (vec) {
-      DISPATCH_T(f32, hipLaunchKernelGGL((glu_act_kernel<T, 4>), dim3(gx, nr), dim3(kThreads), 0, st,
-                                         (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
-                                         out_stride, act));
+      DISPATCH_T(f32, hipLaunchKernelGGL((act_mul_kernel<T, 4>), dim3(gx, nr), dim3(kThreads), 0, st,
+                                         (T*)out + r0 * out_stride, (const T*)gate + r0 * g_stride, g_stride,
+                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act));
     } else {
-      DISPATCH_T(f32, hipLaunchKernelGGL((glu_act_kernel<T, 1>), dim3(gx, nr), dim3(kThreads), 0, st,
-                                         (T*)out + r0 * out_stride, (const T*)gu + r0 * in_stride, F, in_stride,
-                                         out_stride, act));
+      DISPATCH_T(f32, hipLaunchKernelGGL((act_mul_kernel<T, 1>), dim3(gx, nr), dim3(kThreads), 0, st,
+                                         (T*)out + r0 * out_stride, (const T*)gate + r0 * g_stride, g_stride,
+                                         up ? (const T*)up + r0 * u_stride : nullptr, u_stride, F, out_stride, act));
     }
   }
   DX_CHECK_LAUNCH();
@@ -337,15 +548,17 @@ int dxm_glu_act(void* out, const void* gu, int rows, int F, int64_t in_stride, i
 
 int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int64_t* slots, int rows, int n_q, int n_k,
                        int d, int k_off, const float* qw, const float* kw, float eps, float temp_coef,
-                       double temp_every, void* kc, void* vc, int v_mode, int v_off, int v_w, int f32,
-                       hipStream_t st) {
+                       double temp_every, void* kc, void* vc, int v_mode, int v_off, int v_w, const void* v_first,
+                       int64_t vf_stride, float v_lambda, int f32, hipStream_t st) {
   if (rows <= 0) return 0;
   if (n_q < 0 || n_k < 0 || d < 1 || v_mode < 0 || v_mode > 2) return 1;
   if (n_k > 0 && !kc) return 2;
   if (v_mode != 0 && !vc) return 3;
   if (temp_coef != 0.f && !(temp_every > 0)) return 4;
+  if (v_first && v_mode != 2) return 5;
   const int esz = f32 ? 4 : 2;
   const bool vec = d % 4 == 0 && k_off % 4 == 0 && x_stride % 4 == 0 && v_off % 4 == 0 && v_w % 4 == 0 &&
+                   vf_stride % 4 == 0 && (uintptr_t)v_first % (4 * esz) == 0 &&
                    (uintptr_t)x % (4 * esz) == 0 && (uintptr_t)kc % (4 * esz) == 0 && (uintptr_t)vc % (4 * esz) == 0 &&
                    (uintptr_t)qw % 16 == 0 && (uintptr_t)kw % 16 == 0;
   // lanes per head vector: about two chunks of V elements per lane
@@ -355,11 +568,13 @@ int dxm_headprep_cache(void* x, int64_t x_stride, const int64_t* pos, const int6
   if (vec) {
     DISPATCH_T(f32, hipLaunchKernelGGL((headprep_cache_kernel<T, 4>), dim3(rows), dim3(kThreads), 0, st, (T*)x,
                                        x_stride, pos, slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every,
-                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, lpv));
+                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, (const T*)v_first, vf_stride, v_lambda,
+                                       lpv));
   } else {
     DISPATCH_T(f32, hipLaunchKernelGGL((headprep_cache_kernel<T, 1>), dim3(rows), dim3(kThreads), 0, st, (T*)x,
                                        x_stride, pos, slots, n_q, n_k, d, k_off, qw, kw, eps, temp_coef, temp_every,
-                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, lpv));
+                                       (T*)kc, (T*)vc, v_mode, v_off, v_w, (const T*)v_first, vf_stride, v_lambda,
+                                       lpv));
   }
   DX_CHECK_LAUNCH();
   return 0;

@@ -16,6 +16,11 @@
 // activations; with fp32 output (and in the decode kernel) as a bf16 pair
 // hi + lo (two MFMAs), which keeps 16 mantissa bits of every weight.
 //
+// Optional score terms (uniform per launch): a tanh cap, s <- cap tanh(s / cap),
+// and a per-head penalty r1 ln(1 + r2 (p - j)) that grows with the logarithm of
+// the distance; both are applied per element in fp32 before the softmax, in
+// log2 units (tanh from one exp2 and one reciprocal, the logarithm as v_log).
+//
 // Masks are evaluated per element in sequence positions: causal, sliding
 // window (p - size < j <= p) and chunked (floor(j / size) == floor(p / size)),
 // so a prompt cut anywhere gives the same result as one cut nowhere.
@@ -42,7 +47,18 @@ struct TileArgs {
   int Wk, Wv;
   float scale;
   int mask, size;
+  float softcap;    // 0: none
+  const float* r1;  // [n_qh], null: no distance penalty
+  const float* r2;
 };
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// cap * tanh(s / cap) * log2(e) for s in natural units: tanh(x) = 1 - 2 / (1 + e^(2x))
+__device__ __forceinline__ float capped_log2(float s, float cap, float inv_cap) {
+  const float e = fast_exp2(s * (2.f * kLog2e) * inv_cap);
+  return cap * kLog2e * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e));
+}
 
 // positions are < 2^31: 32-bit arithmetic in the kernels
 __device__ __forceinline__ int first_visible(int p, int mask, int size) {
@@ -199,7 +215,10 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
     }
   }
   const bool wave_on = 32 * w < n;
-  const float sc2 = a.scale * 1.4426950408889634f;  // scores in log2 units: exp2 is one instruction
+  const bool terms = a.softcap > 0.f || a.r1 != nullptr;
+  const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  const float r1 = a.r1 ? a.r1[qh] : 0.f, r2 = a.r1 ? a.r2[qh] : 0.f;
+  const float sc2 = terms ? 1.f : a.scale * kLog2e;  // scores in log2 units: exp2 is one instruction
   float mx[2] = {-INFINITY, -INFINITY}, lsum[2] = {0.f, 0.f};
   f32x4 O[2][DVB];
 #pragma unroll
@@ -234,6 +253,22 @@ __global__ void __launch_bounds__(256, (DB + DVB <= 16 ? 2 : 1)) tile_attention_
             S[1][kb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, qf[1][ks], S[1][kb], 0, 0, 0);
           }
         }
+      }
+      if (terms) {  // final scores in log2 units; the exponent's multiplier becomes 1
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+          for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float s2 = S[qb][kb][i] * a.scale;
+              s2 = cap > 0.f ? capped_log2(s2, cap, inv_cap) : s2 * kLog2e;
+              if (a.r1) {
+                const int dist = prow[qb] - (kt + kb * 16 + 4 * g4 + i);
+                s2 -= r1 * __builtin_amdgcn_logf(1.f + r2 * (float)(dist > 0 ? dist : 0));
+              }
+              S[qb][kb][i] = s2;
+            }
       }
       // a tile every row of the wave sees whole needs no per-element mask
       const bool full = 32 * w + 31 < n && kt + kKeys - 1 <= p0 + 32 * w &&
@@ -351,6 +386,9 @@ struct GroupArgs {
   int Wk, Wv;
   float scale;
   int mask, size, parts;
+  float softcap;
+  const float* r1;
+  const float* r2;
 };
 
 template <int DB, int DVB, int QB>
@@ -375,11 +413,15 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
   i16x4 qf[QB][DB];
   bool okh[QB];
   int qh[QB];
+  float r1[QB], r2[QB];
+  const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int hi_ = chunk * 16 * QB + 16 * qb + c16;
     okh[qb] = hi_ < a.group;
     qh[qb] = (g * a.group + (okh[qb] ? hi_ : 0)) * a.maps + m;
+    r1[qb] = a.r1 ? a.r1[qh[qb]] : 0.f;
+    r2[qb] = a.r1 ? a.r2[qh[qb]] : 0.f;
     const bf16_t* q = a.q + (int64_t)row * a.q_stride + (int64_t)qh[qb] * d + 4 * g4;
 #pragma unroll
     for (int ks = 0; ks < DB; ++ks)
@@ -433,7 +475,10 @@ __global__ void __launch_bounds__(64) group_decode_kernel(GroupArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int kj = kt + kb * 16 + 4 * g4 + i;
-          const float s = kj <= p ? S[qb][kb][i] * a.scale : -INFINITY;
+          float s = S[qb][kb][i] * a.scale;
+          if (cap > 0.f) s = cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * s * inv_cap)));
+          if (a.r1) s -= r1[qb] * __logf(1.f + r2[qb] * (float)(p - kj > 0 ? p - kj : 0));
+          s = kj <= p ? s : -INFINITY;
           S[qb][kb][i] = s;
           mloc = fmaxf(mloc, s);
         }
@@ -557,14 +602,15 @@ int dxm_tile_attention_ok(int d, int dv) {
 
 int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
                        const int* seq, const int* bt, int bt_stride, int bs, const int* tiles, int n_tiles, int n_qh,
-                       int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask, int size, int out_f32,
-                       hipStream_t st) {
+                       int maps, int group, int d, int dv, int Wk, int Wv, float scale, int mask, int size,
+                       float softcap, const float* r1, const float* r2, int out_f32, hipStream_t st) {
   if (n_tiles <= 0) return 0;
+  if (softcap < 0.f || (r1 && !r2)) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || n_qh > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || !(scale > 0.f)) return 3;
   if (!seq || !tiles || Wk % 8 || Wv % 8 || q_stride % 8) return 4;
   TileArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, out, pos, seq, bt, bt_stride, bs,
-             tiles, n_qh, maps, group, Wk, Wv, scale, mask, size};
+             tiles, n_qh, maps, group, Wk, Wv, scale, mask, size, softcap, r1, r2};
   TILE_CASE(2, 2)
   TILE_CASE(3, 3)
   TILE_CASE(3, 6)
@@ -583,13 +629,15 @@ int dxm_tile_attention(void* out, const void* q, int64_t q_stride, const void* k
 // [rows, n_qh, parts, 2 + dv]; dxm_merge_parts joins them.
 int dxm_group_decode(float* ws, const void* q, int64_t q_stride, const void* kc, const void* vc, const int64_t* pos,
                      const int* seq, const int* bt, int bt_stride, int bs, int rows, int n_qh, int maps, int group,
-                     int d, int dv, int Wk, int Wv, float scale, int mask, int size, int parts, hipStream_t st) {
+                     int d, int dv, int Wk, int Wv, float scale, int mask, int size, float softcap, const float* r1,
+                     const float* r2, int parts, hipStream_t st) {
   if (rows <= 0) return 0;
+  if (softcap < 0.f || (r1 && !r2)) return 6;
   if (n_qh < 1 || maps < 1 || group < 1 || n_qh % maps || (n_qh / maps) % group || rows > 65535) return 1;
   if (mask < 0 || mask > 2 || (mask && size < 1) || parts < 1 || parts > 65535) return 3;
   if (!ws || Wk % 8 || Wv % 8 || q_stride % 4) return 4;
   GroupArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, ws, pos, seq, bt, bt_stride, bs,
-              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts};
+              n_qh, maps, group, 1, Wk, Wv, scale, mask, size, parts, softcap, r1, r2};
   GROUP_CASE(2, 2)
   GROUP_CASE(3, 3)
   GROUP_CASE(3, 6)

@@ -98,11 +98,14 @@ def expert(h, W, pre):
     return (g * torch.sigmoid(g) * (h @ W[pre + "up"].T)) @ W[pre + "down"].T
 
 
-def route(z, correction, top, groups):
-    """Per token: chosen experts [T, top] and their weights.  z [T, E] router logits."""
+def route(z, correction, top, groups, margin=None):
+    """Per token: chosen experts [T, top] and their weights.  z [T, E] router logits.
+    margin (a list): gets a [T] tensor, how far each token's choice is from another one
+    (the gap between the last score taken and the first one left, of groups and of experts)."""
     s = torch.sigmoid(z)
     c = s + correction
     T, E = c.shape
+    gap = torch.full((T,), float("inf"), dtype=c.dtype)
     if groups:
         n, keep = groups["count"], groups["keep"]
         per = E // n
@@ -110,14 +113,22 @@ def route(z, correction, top, groups):
         gs = cg.topk(min(2, per), -1).values.sum(-1)
         kept = torch.zeros(T, n, dtype=torch.bool)
         kept.scatter_(1, gs.topk(keep, -1).indices, True)
+        if keep < n:
+            g = gs.sort(-1, descending=True).values
+            gap = g[:, keep - 1] - g[:, keep]
         c = c.masked_fill(~kept[:, :, None].expand(T, n, per).reshape(T, E), float("-inf"))
     idx = c.topk(top, -1).indices
+    if top < E:
+        cs = c.sort(-1, descending=True).values
+        gap = torch.minimum(gap, cs[:, top - 1] - cs[:, top])
+    if margin is not None:
+        margin.append(gap)
     return idx, s.gather(1, idx)
 
 
-def ff_moe(h, W, pre, mlp):
+def ff_moe(h, W, pre, mlp, margin=None):
     r = mlp["router"]
-    idx, wgt = route(h @ W[pre + "router"].T, W[pre + "correction"], r["top"], r.get("groups"))
+    idx, wgt = route(h @ W[pre + "router"].T, W[pre + "correction"], r["top"], r.get("groups"), margin)
     out = torch.zeros(h.shape[0], W[pre + "e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
         for e, w in zip(idx[t].tolist(), wgt[t]):
@@ -135,7 +146,7 @@ def token_side(x, W, i, toks, dim, eps):
     return x + unit_rms(y, eps) * W[f"l{i}.side.norm"]
 
 
-def forward(cfg: dict, W: dict, toks, return_layers: bool = False):
+def forward(cfg: dict, W: dict, toks, return_layers: bool = False, margin: list | None = None):
     W = {k: (v.to(F) if v.is_floating_point() else v) for k, v in W.items()}
     eps = cfg["norm"]["eps"]
     toks = torch.as_tensor(toks, dtype=torch.long)
@@ -149,7 +160,7 @@ def forward(cfg: dict, W: dict, toks, return_layers: bool = False):
             v_first = v_own
         mlp = L.get("mlp")
         if mlp:
-            y = y + (ff_dense(h, W, f"l{i}.mlp.") if mlp["kind"] == "dense" else ff_moe(h, W, f"l{i}.mlp.", mlp))
+            y = y + (ff_dense(h, W, f"l{i}.mlp.") if mlp["kind"] == "dense" else ff_moe(h, W, f"l{i}.mlp.", mlp, margin))
         x = x + y
         if cfg.get("token_side"):
             x = token_side(x, W, i, toks, cfg["token_side"]["dim"], eps)
