@@ -1,5 +1,6 @@
-"""`bench.py --layered`: a layer-listed model (Bekulix) beside the closest
-existing model (Llama) at equal layer sizes, random weights.
+"""`bench.py --layered`: the layer-listed models (Bekulix, Bolinex) beside the
+closest existing model (Llama) at equal layer sizes, random weights.
+`--layered-family` picks which of the two families runs (default both).
 
 Two parts, both on one GPU:
   * engine throughput through the engine's own entry point (add_request +
@@ -14,6 +15,7 @@ Two parts, both on one GPU:
 from __future__ import annotations
 
 import math
+import sys
 import time
 
 import torch
@@ -21,8 +23,9 @@ import torch
 from .. import ops
 from ..engine.engine import EngineConfig, LLMEngine
 from ..engine.request import SamplingParams
-from ..models.config import ModelConfig, _bekulix_preset
+from ..models.config import ModelConfig, _bekulix_preset, _bolinex_preset
 from ..ops import mixers as mx
+from ..ops import moe
 
 # layer sizes of real models (width, ff, heads, kv heads, head dim), a few layers each
 SIZES = {
@@ -38,6 +41,14 @@ def _configs(s: dict):
                       num_hidden_layers=s["layers"], num_attention_heads=s["H"], num_key_value_heads=s["G"],
                       head_dim=s["d"], max_position_embeddings=8192, bos_token_id=1, eos_token_id=[2])
     return bek, lla
+
+
+def _bolinex_config(s: dict):
+    """Bolinex at the size's layer shapes: window 1024, every second feed-forward 8 experts of a
+    quarter of the dense width (two chosen, in two of four groups) plus a shared one."""
+    return _bolinex_preset(f"bolinex {s['W']}", s["W"], s["ff"], s["layers"], s["H"], s["G"], s["d"], 1024, experts=8,
+                           top=2, expert_ff=s["ff"] // 4, shared_ff=s["ff"] // 4, groups=(4, 2), side=256,
+                           vocab=s["vocab"])
 
 
 def _timed(fn, iters=10, warm=2) -> float:
@@ -57,6 +68,7 @@ def engine_throughput(mcfg, dev, isl: int, osl: int, prefill_seqs: int, decode_s
     out = {}
     g = torch.Generator().manual_seed(seed)
     for phase, B in (("prefill", prefill_seqs), ("decode", decode_seqs)):
+        print(f"[layered] {mcfg.name}: {phase}", file=sys.stderr, flush=True)
         eng = LLMEngine(EngineConfig(model=mcfg.name, device=str(dev), block_size=64, max_model_len=isl + osl + 64,
                                      max_num_seqs=B, max_num_batched_tokens=max(8192, prefill_seqs * isl),
                                      chunked_prefill=False, max_prefill_streak=1 << 30, enable_prefix_caching=False,
@@ -192,17 +204,119 @@ def rowwise_kernels(s: dict, T: int) -> dict:
     return res
 
 
+def bolinex_kernels(s: dict, L: int, B: int, T: int) -> dict:
+    """Bolinex's kernels alone, each beside its counterpart: window attention with the score
+    cap and the distance penalty against the same kernels without them (prefill in TFLOP/s of
+    the visible scores, decode in TB/s of the window's cache bytes); the residual step with a
+    layer norm against Llama's add + RMS norm; the gate product; routing, plan and the grouped
+    GEMMs of one routed feed-forward against one dense GEMM pair of the same FLOPs."""
+    H, G, d, W, ff, bs = s["H"], s["G"], s["d"], s["W"], s["ff"], 64
+    dev, dt, win = "cuda", torch.bfloat16, 1024
+    res = {}
+    nb = L // bs + 1
+    q = torch.randn(L, H * d, device=dev, dtype=dt)
+    pos = torch.arange(L, device=dev)
+    seq = torch.zeros(L, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(1, nb)
+    kc = torch.randn(nb * bs, G * d, device=dev, dtype=dt)
+    vc = torch.randn_like(kc)
+    tiles = torch.tensor(mx.tile_list(0, L), dtype=torch.int32, device=dev)
+    r1 = torch.rand(H, device=dev)
+    r2 = torch.rand(H, device=dev) + 0.1
+    j = torch.arange(L)
+    fl = 4 * d * H * float((j - mx.first_visible(j, "window", win) + 1).sum())
+    for name, kw in (("plain", {}), ("cap", dict(softcap=30.0)), ("cap_penalty", dict(softcap=30.0, dist_bias=(r1, r2)))):
+        us = _timed(lambda: mx.attention(q, kc, vc, pos, seq, bt, bs, H, 1, H // G, d, d, d ** -0.5, "window", win, 1,
+                                         False, tiles, L, **kw))
+        res[f"prefill_window{win}_{name}"] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1)}
+    nbb = B * nb
+    byts = B * min(L, win) * G * d * 2 * 2
+    btd = torch.randperm(nbb, device=dev).to(torch.int32).view(B, nb)
+    kcd = torch.randn(nbb * bs, G * d, device=dev, dtype=dt)
+    vcd = torch.randn_like(kcd)
+    qd = torch.randn(B, H * d, device=dev, dtype=dt)
+    posd = torch.full((B,), L - 1, device=dev)
+    parts = mx.row_attention_parts(B, G, win)
+    for name, kw in (("plain", {}), ("cap_penalty", dict(softcap=30.0, dist_bias=(r1, r2)))):
+        us = _timed(lambda: mx.attention(qd, kcd, vcd, posd, None, btd, bs, H, 1, H // G, d, d, d ** -0.5, "window", win,
+                                         parts, **kw))
+        res[f"decode_window{win}_{name}"] = {"us": round(us, 1), "TB/s": round(byts / us / 1e6, 2), "parts": parts}
+
+    def put(name, us, byts=None, flops=None):
+        res[name] = {"us": round(us, 1)}
+        if byts:
+            res[name]["TB/s"] = round(byts / us / 1e6, 2)
+        if flops:
+            res[name]["TFLOPs"] = round(flops / us / 1e6, 1)
+
+    X = torch.randn(T, W, device=dev)
+    a, b, c = (torch.randn(T, W, device=dev, dtype=dt) for _ in range(3))
+    nw = torch.ones(W, device=dev)
+    put("residual_step_two_addends_layernorm",
+        _timed(lambda: mx.residual_step(X, a, b, eps=1e-5, norm="layer", norm_w=nw, norm_b=nw, out_dtype=dt)),
+        T * W * (4 + 4 + 2 + 2 + 2))
+    put("residual_step_unit_rms_addend_layernorm",
+        _timed(lambda: mx.residual_step(X, c=c, c_w=nw, eps=1e-5, norm="layer", norm_w=nw, norm_b=nw, out_dtype=dt)),
+        T * W * (4 + 4 + 2 + 2))
+    r = torch.randn(T, W, device=dev, dtype=dt)
+    w16 = torch.ones(W, device=dev, dtype=dt)
+    put("llama_add_rmsnorm", _timed(lambda: ops.add_rmsnorm(a, r, w16, 1e-6)), T * W * 2 * 4)
+    p = torch.randn(T, 2 * H * d, device=dev, dtype=dt)
+    put("act_mul_sigmoid_gate", _timed(lambda: mx.act_mul(p[:, H * d:], p[:, :H * d], "sigmoid")), T * H * d * 2 * 3)
+    u = torch.randn(T, ff, device=dev, dtype=dt)
+    put("act_mul_relu2", _timed(lambda: mx.act_mul(u, None, "relu2")), T * ff * 2 * 2)
+    gu = torch.randn(T, 2 * ff, device=dev, dtype=dt)
+    put("llama_silu_and_mul", _timed(lambda: ops.silu_and_mul(gu)), T * ff * 2 * 3)
+    # one routed feed-forward: E experts of width ff / 4, two per token
+    E, top, fe = 8, 2, ff // 4
+    for rows, tag in ((T, "prefill"), (B, "decode")):
+        h = torch.randn(rows, W, device=dev, dtype=dt)
+        z = torch.randn(rows, E, device=dev)
+        corr = torch.zeros(E, device=dev)
+        put(f"moe_route_{tag}", _timed(lambda: moe.route(z, corr, top, 4, 2)))
+        idx, wgt = moe.route(z, corr, top, 4, 2)
+        put(f"moe_plan_{tag}", _timed(lambda: moe.plan(idx, E)))
+        order, offsets = moe.plan(idx, E)
+        wgu = torch.randn(E, 2 * fe, W, device=dev, dtype=dt) * W ** -0.5
+        wdn = torch.randn(E, W, fe, device=dev, dtype=dt) * fe ** -0.5
+        f1, f2 = 2.0 * rows * top * W * 2 * fe, 2.0 * rows * top * fe * W
+        # decode: the weights of the experts in use are what has to move
+        used = int((offsets[1:] > offsets[:-1]).sum())
+        wb1, wb2 = used * 2 * fe * W * 2, used * W * fe * 2
+        put(f"grouped_gemm_gate_up_{tag}", _timed(lambda: moe.grouped_gemm(h, wgu, order, offsets, top, True, False)),
+            wb1 if tag == "decode" else None, f1)
+        act = torch.randn(rows * top, fe, device=dev, dtype=dt)
+        put(f"grouped_gemm_down_{tag}", _timed(lambda: moe.grouped_gemm(act, wdn, order, offsets, top, False, True)),
+            wb2 if tag == "decode" else None, f2)
+        # the library's dense GEMMs of the same FLOPs (rows * top rows against one expert's weights)
+        hd = torch.randn(rows * top, W, device=dev, dtype=dt)
+        put(f"dense_gemm_gate_up_{tag}", _timed(lambda: torch.matmul(hd, wgu[0].t())),
+            2 * fe * W * 2 if tag == "decode" else None, f1)
+        put(f"dense_gemm_down_{tag}", _timed(lambda: torch.matmul(act, wdn[0].t())),
+            W * fe * 2 if tag == "decode" else None, f2)
+        y = torch.randn(rows * top, W, device=dev, dtype=dt)
+        sh = torch.randn(rows, W, device=dev, dtype=dt)
+        put(f"moe_combine_{tag}", _timed(lambda: moe.combine(y, wgt, sh)), rows * W * 2 * (top + 2))
+    return res
+
+
 def run_layered_compare(args, dev) -> dict:
     isl, osl = min(args.isl, 2048), min(args.osl, 64)
+    fam = getattr(args, "layered_family", "all")
     sizes = {}
     for name, s in SIZES.items():
         bek, lla = _configs(s)
         row = {"layers": s["layers"], "isl": isl, "osl": osl, "prefill_seqs": 4, "decode_seqs": 64}
-        row["bekulix"] = engine_throughput(bek, dev, isl, osl, 4, 64, args.seed)
+        if fam in ("all", "bekulix"):
+            row["bekulix"] = engine_throughput(bek, dev, isl, osl, 4, 64, args.seed)
+        if fam in ("all", "bolinex"):
+            row["bolinex"] = engine_throughput(_bolinex_config(s), dev, isl, osl, 4, 64, args.seed)
+            row["bolinex_kernels"] = bolinex_kernels(s, 4096, 64, 8192)
         row["llama"] = engine_throughput(lla, dev, isl, osl, 4, 64, args.seed)
         row["attention_kernels"] = attention_kernels(s, 4096, 64)
-        row["rowwise_kernels"] = rowwise_kernels(s, 8192)
+        if fam in ("all", "bekulix"):
+            row["rowwise_kernels"] = rowwise_kernels(s, 8192)
         sizes[name] = row
-    return {"metric": "layer-listed model (Bekulix) beside Llama at equal layer sizes: engine prefill / decode "
-                      "tokens/s and attention kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
-            "data": "synthetic (random-token prompts, random-init weights)", "sizes": sizes}
+    return {"metric": "layer-listed models (Bekulix, Bolinex) beside Llama at equal layer sizes: engine prefill / "
+                      "decode tokens/s and kernels alone", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+            "family": fam, "data": "synthetic (random-token prompts, random-init weights)", "sizes": sizes}
