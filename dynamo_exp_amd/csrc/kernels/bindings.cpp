@@ -28,6 +28,8 @@ int dx_kv_dequant(const void*, const void*, void*, void*, const int*, int, const
 int dx_kv_write(const void*, const void*, int64_t, const int64_t*, void*, void*, int, int, int, int, hipStream_t);
 int dx_silu_and_mul(void*, const void*, int, int, int64_t, int64_t, int, hipStream_t);
 int dx_gemm256(void*, int64_t, const void*, int64_t, const void*, int, int, int, int, int, hipStream_t, const float*);
+int dx_gemm256_grouped(void*, int64_t, const void*, int64_t, int64_t, const void*, const int*, const int*, int, int,
+                       int, int, int, int, int, int, int, hipStream_t);
 int dx_row_rrms(float*, const void*, int, int, int64_t, float, hipStream_t);
 int dx_embedding(void*, const void*, const void*, int, int, int, int64_t, hipStream_t);
 int dx_decode_attention(void*, float*, float*, const void*, int64_t, const void*, const void*, const int*, int,
@@ -128,6 +130,12 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("prefill_tile_tokens", &dx_prefill_tile_tokens);
   m.def("gemm256", [](u y, int64_t ldy, u x, int64_t ldx, u w, int M, int N, int K, int epi, int gm, u st, u rs) {
     check(dx_gemm256(P(y), ldy, P(x), ldx, P(w), M, N, K, epi, gm, S(st), (const float*)rs), "gemm256");
+  });
+  m.def("gemm256_grouped", [](u y, int64_t ldy, u x, int64_t ldx, int64_t x_rows, u w, u order, u offsets, int R, int E,
+                              int N, int K, int top, int gather, int scatter, int epi, int gm, u st) {
+    check(dx_gemm256_grouped(P(y), ldy, P(x), ldx, x_rows, P(w), (const int*)order, (const int*)offsets, R, E, N, K, top,
+                             gather, scatter, epi, gm, S(st)),
+          "gemm256_grouped");
   });
   m.def("skinny_gemm", [](u y, int64_t ys, u x, int64_t xs, u w, u slabs, u tickets, int M, int N, int K, int bn,
                           int bm, int splits, u st) {

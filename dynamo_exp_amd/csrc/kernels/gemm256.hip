@@ -35,6 +35,13 @@
 //     group's refill one phase later cannot overtake the lagging group's reads;
 //     the DMA waits sit at the end of each phase and cover the parts read two
 //     phases later (one barrier before the lagging group reads them).
+//   * Grouped mode (mixture of experts): the token rows are sorted by expert
+//     (order / offsets, built on the device), an expert's run of rows is cut
+//     into 256-row tiles against that expert's weight matrix w[e] (w is
+//     [E, N, K]), x rows are gathered per lane (the DMA takes any row address)
+//     and y rows scattered by the same map.  The host does not know the
+//     experts' row counts: the grid walks an upper bound of row tiles and
+//     every workgroup skips the ones past the last expert.
 //   * Blocks are remapped so that each XCD walks a contiguous range of tiles
 //     (bijective for any grid size), in bands of group_m token tiles: the ~32
 //     workgroups resident on one XCD then share group_m x tiles and
@@ -60,11 +67,19 @@ enum { EPI_STORE = 0, EPI_SILU = 1, EPI_SILU_RS = 2 };
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.f + __expf(-g)); }
 
-template <int EPI>
+// Grouped mode: sorted row r (offsets[e] <= r < offsets[e + 1] belongs to expert e)
+// reads x row order[r] / top (gather) or r, and writes y row order[r] (scatter) or r.
+struct GroupMap {
+  const int* order;
+  const int* offsets;
+  int E, top, gather, scatter;
+};
+
+template <int EPI, bool GRP>
 __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, int64_t ldy,
                                                       const bf16_t* __restrict__ x, int64_t ldx,
                                                       const bf16_t* __restrict__ w, int M, int N, int K,
-                                                      int group_m, const float* __restrict__ rs) {
+                                                      int group_m, const float* __restrict__ rs, GroupMap gm) {
   __shared__ __attribute__((aligned(16))) char smem[kLds];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -74,7 +89,8 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
   // ---- persistent, XCD-aware tile order: the workgroups on one XCD (blocks
   // b, b + 8, ...) walk one contiguous range of logical tiles, stride = their
   // count, so the ~32 tiles in flight on an XCD are always neighbours
-  const int mtn = (M + kBM - 1) / kBM, ntn = N / kBN, nwg = mtn * ntn;
+  // grouped: M is the number of sorted rows; at most this many row tiles over all experts
+  const int mtn = (M + kBM - 1) / kBM + (GRP ? gm.E : 0), ntn = N / kBN, nwg = mtn * ntn;
   const int G = gridDim.x, bid = blockIdx.x, xcd = bid & 7;
   const int gq = G >> 3, gr8 = G & 7;                 // workgroups on this XCD: gq (+1)
   const int per_xcd = xcd < gr8 ? gq + 1 : gq;
@@ -193,11 +209,37 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
   // workgroup and K-step through the XCD's L2 instead of 33 KB for one weight
   // tile x 32 token tiles)
   int mt = 0, nt = 0;
-  auto select = [&](int lid) {
+  int row0 = 0, rend = 0;  // grouped: this tile's first sorted row and its expert's end
+  // false (grouped only): the row tile lies past the last expert's rows
+  auto select = [&](int lid) -> bool {
     const int band = lid / (group_m * ntn), first_m = band * group_m;
     const int gsz = min(mtn - first_m, group_m), in_band = lid - band * group_m * ntn;
     mt = first_m + in_band % gsz;
     nt = in_band / gsz;
+    if constexpr (GRP) {
+      int e = 0, rem = mt, lo = 0, hi = 0;
+      for (; e < gm.E; ++e) {
+        lo = gm.offsets[e];
+        hi = gm.offsets[e + 1];
+        const int n = (hi - lo + kBM - 1) / kBM;
+        if (rem < n) break;
+        rem -= n;
+      }
+      if (e >= gm.E) return false;
+      row0 = lo + rem * kBM;
+      rend = hi;
+      xb = x;
+      wb = w + ((int64_t)e * N + (int64_t)nt * kBN) * K;
+#pragma unroll
+      for (int P = 0; P < 2; ++P)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int r = min(row0 + prow[P][i], rend - 1);
+          const int src = gm.gather ? gm.order[r] / gm.top : r;
+          xoff[P][i] = src * (int)ldx + goff[P][i];
+        }
+      return true;
+    }
     xb = x + (int64_t)mt * kBM * ldx;
     wb = w + (int64_t)nt * kBN * K;
 #pragma unroll
@@ -205,6 +247,13 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
 #pragma unroll
       for (int i = 0; i < 2; ++i)
         xoff[P][i] = (min(mt * kBM + prow[P][i], M - 1) - mt * kBM) * (int)ldx + goff[P][i];
+    return true;
+  };
+  // the first tile at or after lid (in this workgroup's stride) that exists; t_end if none
+  auto next_tile = [&](int from) -> int {
+    for (int l = from; l < t_end; l += per_xcd)
+      if (select(l)) return l;
+    return t_end;
   };
   // prologue of a tile: tile 0 of K, then K-tile 1 without its x half 1 (issued in p1 of K-tile 0)
   auto prologue = [&]() {
@@ -217,9 +266,8 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
     issue(3, 1, 1);
   };
 
-  int lid = t_begin + (bid >> 3);
+  int lid = next_tile(t_begin + (bid >> 3));
   if (lid >= t_end) return;
-  select(lid);
   prologue();
   for (;;) {
 #pragma unroll
@@ -240,7 +288,16 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped tail reloads landed before the buffers are refilled
 
     const int cmt = mt, cnt = nt;
-    const int tok0 = cmt * kBM + wr * 128 + l15;
+    const int tok0 = (GRP ? row0 : cmt * kBM) + wr * 128 + l15;
+    const int tok_end = GRP ? rend : M;
+    // grouped + scatter: the 8 destination rows, loaded and retired like the row scales below
+    int dstv[8];
+    if constexpr (GRP) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dstv[j] = gm.scatter ? gm.order[min(tok0 + 16 * j, tok_end - 1)] : tok0 + 16 * j;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) asm volatile("" ::"v"(dstv[j]));
+    }
     // EPI_SILU_RS: the 8 row scales this lane needs, loaded in one batch and
     // retired BEFORE the next tile's prologue DMA is queued (the empty asm
     // consumes them): vmcnt retires in order, and the compiler otherwise
@@ -255,11 +312,10 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
     }
 
     // the next tile's first K-tiles go out before this tile's stores
-    const int nlid = lid + per_xcd;
+    const int nlid = next_tile(lid + per_xcd);
     const bool more = nlid < t_end;
     if (more) {
       lid = nlid;
-      select(lid);
       prologue();
     }
 
@@ -268,8 +324,8 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int tok = tok0 + 16 * j;
-        if (tok >= M) continue;
-        bf16_t* yr = y + (int64_t)tok * ldy + cnt * kBN + wc * 64 + 4 * lq;
+        if (tok >= tok_end) continue;
+        bf16_t* yr = y + (int64_t)(GRP ? dstv[j] : tok) * ldy + cnt * kBN + wc * 64 + 4 * lq;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           uint2 pk;
@@ -282,8 +338,8 @@ __global__ void __launch_bounds__(512) gemm256_kernel(bf16_t* __restrict__ y, in
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int tok = tok0 + 16 * j;
-        if (tok >= M) continue;
-        bf16_t* yr = y + (int64_t)tok * ldy + cnt * (kBN / 2) + wc * 32 + 4 * lq;
+        if (tok >= tok_end) continue;
+        bf16_t* yr = y + (int64_t)(GRP ? dstv[j] : tok) * ldy + cnt * (kBN / 2) + wc * 32 + 4 * lq;
         const float sc = EPI == EPI_SILU_RS ? scv[j] : 1.f;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -323,7 +379,16 @@ void launch(bf16_t* y, int64_t ldy, const bf16_t* x, int64_t ldx, const bf16_t* 
             int persistent, hipStream_t st, const float* rs) {
   const int tiles = ((M + kBM - 1) / kBM) * (N / kBN);
   const int grid = persistent ? std::min(tiles, num_cus()) : tiles;
-  hipLaunchKernelGGL((gemm256_kernel<EPI>), dim3(grid), dim3(512), 0, st, y, ldy, x, ldx, w, M, N, K, gm, rs);
+  hipLaunchKernelGGL((gemm256_kernel<EPI, false>), dim3(grid), dim3(512), 0, st, y, ldy, x, ldx, w, M, N, K, gm, rs,
+                     GroupMap{nullptr, nullptr, 0, 1, 0, 0});
+}
+
+template <int EPI>
+void launch_grouped(bf16_t* y, int64_t ldy, const bf16_t* x, int64_t ldx, const bf16_t* w, int R, int N, int K, int gm,
+                    hipStream_t st, const GroupMap& map) {
+  const int tiles = ((R + kBM - 1) / kBM + map.E) * (N / kBN);
+  hipLaunchKernelGGL((gemm256_kernel<EPI, true>), dim3(std::min(tiles, num_cus())), dim3(512), 0, st, y, ldy, x, ldx, w,
+                     R, N, K, gm, nullptr, map);
 }
 
 }  // namespace
@@ -349,6 +414,31 @@ extern "C" int dx_gemm256(void* y, int64_t ldy, const void* x, int64_t ldx, cons
   if (epi == EPI_STORE) launch<EPI_STORE>(Y, ldy, X, ldx, W, M, N, K, group_m, persistent, st, nullptr);
   else if (epi == EPI_SILU) launch<EPI_SILU>(Y, ldy, X, ldx, W, M, N, K, group_m, persistent, st, nullptr);
   else if (epi == EPI_SILU_RS && rs != nullptr) launch<EPI_SILU_RS>(Y, ldy, X, ldx, W, M, N, K, group_m, persistent, st, rs);
+  else return 2;
+  DX_CHECK_LAUNCH();
+  return 0;
+}
+
+// Grouped GEMM over the rows of each expert: w [E, N, K]; order [R] / offsets [E + 1]
+// sort the R rows by expert (see GroupMap).  epi 0: y[dst, N]; epi 1: SwiGLU over 32-row
+// interleaved gate/up rows of every w[e], y[dst, N/2].  x_rows: rows of x (its row
+// addresses must fit 32-bit element offsets).  Same shape requirements as dx_gemm256.
+extern "C" int dx_gemm256_grouped(void* y, int64_t ldy, const void* x, int64_t ldx, int64_t x_rows, const void* w,
+                                  const int* order, const int* offsets, int R, int E, int N, int K, int top,
+                                  int gather, int scatter, int epi, int group_m, hipStream_t st) {
+  if (R < 1) return 0;
+  if (E < 1 || top < 1 || group_m < 1 || !order || !offsets) return 7;
+  if (N % kBN != 0 || K % (2 * kBK) != 0 || K < 2 * kBK) return 3;
+  if ((ldx & 7) || (ldy & 3) || (reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(w) & 15) ||
+      (reinterpret_cast<uintptr_t>(y) & 7))
+    return 5;
+  if ((int64_t)N * K >= (1ll << 31) || x_rows * ldx >= (1ll << 31)) return 6;  // 32-bit DMA offsets
+  const GroupMap map{order, offsets, E, top, gather, scatter};
+  auto* Y = static_cast<bf16_t*>(y);
+  auto* X = static_cast<const bf16_t*>(x);
+  auto* W = static_cast<const bf16_t*>(w);
+  if (epi == EPI_STORE) launch_grouped<EPI_STORE>(Y, ldy, X, ldx, W, R, N, K, group_m, st, map);
+  else if (epi == EPI_SILU) launch_grouped<EPI_SILU>(Y, ldy, X, ldx, W, R, N, K, group_m, st, map);
   else return 2;
   DX_CHECK_LAUNCH();
   return 0;

@@ -236,10 +236,15 @@ class BolinexForCausalLM:
                 out.update(w_up=act(q + "up"), w_down=act(q + "down"))
             elif mlp:
                 E = mlp["router"]["experts"]
+                w_egu = torch.stack([torch.cat([sd[f"{q}e{e}.gate"], sd[f"{q}e{e}.up"]], 0)
+                                     for e in range(E)]).to(dev, dt).contiguous()
+                # where the 256-tile GEMM serves the shape, gate and up rows are interleaved
+                # for its SwiGLU epilogue and the [rows, 2 ff] intermediate is never written
+                probe = torch.empty((1, w_egu.shape[2]), device=dev, dtype=dt)
+                fused = moe.tile_gemm_ok(probe, w_egu) and (w_egu.shape[1] // 2) % moe.GLU_BLOCK == 0
                 out.update(router=f32(sd[q + "router"]),
                            correction=f32(sd[q + "correction"]) if q + "correction" in sd else None,
-                           w_egu=torch.stack([torch.cat([sd[f"{q}e{e}.gate"], sd[f"{q}e{e}.up"]], 0)
-                                              for e in range(E)]).to(dev, dt).contiguous(),
+                           w_egu=moe.interleave_glu(w_egu) if fused else w_egu, egu_fused=fused,
                            w_edown=torch.stack([sd[f"{q}e{e}.down"] for e in range(E)]).to(dev, dt).contiguous())
                 if mlp.get("shared"):
                     out.update(w_sgu=act(q + "shared.gate", q + "shared.up"), w_sdown=act(q + "shared.down"))
@@ -294,8 +299,12 @@ class BolinexForCausalLM:
         z = torch.matmul(h.float(), L["router"].t())
         idx, w = moe.route(z, L["correction"], r["top"], gr["count"], gr["keep"])
         order, offsets = moe.plan(idx, r["experts"])
-        gu = moe.grouped_gemm(h, L["w_egu"], order, offsets, r["top"], gather=True, scatter=False)
-        y = moe.grouped_gemm(mx.glu_act(gu, "silu"), L["w_edown"], order, offsets, r["top"], gather=False, scatter=True)
+        if L["egu_fused"]:
+            act = moe.grouped_gemm(h, L["w_egu"], order, offsets, r["top"], gather=True, scatter=False, glu=True)
+        else:
+            act = mx.glu_act(moe.grouped_gemm(h, L["w_egu"], order, offsets, r["top"], gather=True, scatter=False),
+                             "silu")
+        y = moe.grouped_gemm(act, L["w_edown"], order, offsets, r["top"], gather=False, scatter=True)
         shared = None
         if "w_sgu" in L:
             shared = torch.matmul(mx.glu_act(torch.matmul(h, L["w_sgu"].t()), "silu"), L["w_sdown"].t())

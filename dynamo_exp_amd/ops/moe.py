@@ -19,7 +19,7 @@ import torch
 from .. import _native
 from .mixers import _f32, _fp32_param, _ptr, _stream
 
-GEMM_TILE_M = 64  # sorted rows per grouped-GEMM workgroup
+GLU_BLOCK = 32  # rows per gate / up block of weights interleaved for the fused SwiGLU epilogue
 
 
 def _m():
@@ -83,13 +83,37 @@ def plan(idx: torch.Tensor, n_experts: int) -> tuple[torch.Tensor, torch.Tensor]
     return order, offsets
 
 
+def tile_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the 256 x 256-tile matrix-core GEMM (csrc/kernels/gemm256.hip, grouped
+    mode) takes a [rows, K] against w [E, N, K]; the 64 x 64-tile kernel of
+    csrc/mixers/moe.hip takes everything else."""
+    E, N, K = w.shape
+    return (a.is_cuda and a.dtype == torch.bfloat16 and N % 256 == 0 and K % 128 == 0 and a.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and N * K < 2 ** 31
+            and a.shape[0] * a.stride(0) < 2 ** 31)
+
+
+def interleave_glu(w: torch.Tensor) -> torch.Tensor:
+    """[E, 2F, K] = per expert [gate | up] rows -> blocks of GLU_BLOCK gate rows followed by
+    their GLU_BLOCK up rows, the layout of the fused SwiGLU epilogue (F % GLU_BLOCK == 0)."""
+    E, F2, K = w.shape
+    F = F2 // 2
+    if F % GLU_BLOCK:
+        raise ValueError("interleave_glu: the expert width must be a multiple of the block")
+    g, u = w[:, :F].view(E, F // GLU_BLOCK, GLU_BLOCK, K), w[:, F:].view(E, F // GLU_BLOCK, GLU_BLOCK, K)
+    return torch.stack([g, u], 2).reshape(E, F2, K).contiguous()
+
+
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, offsets: torch.Tensor, top: int,
-                 gather: bool, scatter: bool) -> torch.Tensor:
+                 gather: bool, scatter: bool, glu: bool = False) -> torch.Tensor:
     """Per expert e, the rows r of its run offsets[e] .. offsets[e + 1] times
     w[e]^T  (w [E, N, K], stored [out, in]).  Row r reads a[order[r] // top]
     when `gather` (a holds one row per token) and a[r] otherwise (a is already
     in sorted order); it is written to out[order[r]] when `scatter` (slot
-    order) and to out[r] otherwise.  Products accumulate in fp32."""
+    order) and to out[r] otherwise.  Products accumulate in fp32.
+    `glu`: w holds gate and up rows interleaved (interleave_glu) and the result
+    is silu(gate) * up, [R, N / 2], formed in the GEMM's epilogue; only where
+    tile_gemm_ok (the caller keeps plain [gate | up] weights otherwise)."""
     E, N, K = w.shape
     R = order.shape[0]
     if a.dtype != w.dtype or a.shape[1] != K or a.stride(1) != 1 or not w.is_contiguous():
@@ -97,6 +121,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, offsets:
     if (not gather and a.shape[0] != R) or (gather and a.shape[0] * top != R):
         raise ValueError("grouped_gemm: row count does not fit the plan")
     if not a.is_cuda:
+        if glu:
+            raise ValueError("grouped_gemm: the fused SwiGLU epilogue is a GPU path")
         out = torch.empty((R, N), dtype=a.dtype)
         o = order.long()
         off = offsets.tolist()
@@ -108,7 +134,14 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, offsets:
         return out
     if order.dtype != torch.int32 or offsets.dtype != torch.int32 or offsets.numel() != E + 1:
         raise TypeError("grouped_gemm: int32 order and offsets [E + 1]")
-    out = torch.empty((R, N), dtype=a.dtype, device=a.device)
+    if glu and not tile_gemm_ok(a, w):
+        raise ValueError("grouped_gemm: the fused SwiGLU epilogue needs tile_gemm_ok operands")
+    out = torch.empty((R, N // 2 if glu else N), dtype=a.dtype, device=a.device)
+    if tile_gemm_ok(a, w):
+        _native.kernels().gemm256_grouped(out.data_ptr(), out.stride(0), a.data_ptr(), a.stride(0), a.shape[0],
+                                          w.data_ptr(), order.data_ptr(), offsets.data_ptr(), R, E, N, K, top,
+                                          int(gather), int(scatter), int(glu), 8, _stream())
+        return out
     _m().grouped_gemm(out.data_ptr(), a.data_ptr(), a.stride(0), w.data_ptr(), order.data_ptr(), offsets.data_ptr(),
                       R, E, N, K, top, int(gather), int(scatter), _f32(a), _stream())
     return out

@@ -88,6 +88,10 @@ CONFIGS = {
                              layer(mixer(H=2, G=1, d=64, dv=64, window=70), experts(E=8, top=2, ff=32, shared=32)),
                              layer(mixer(H=4, G=2, d=48, dv=96, window=33, v_mix=False), dense(64)),
                              layer(mixer(H=2, G=1, d=64, dv=64, window=0, cap=0), None)], width=64, side=8),
+    # expert shapes the 256-tile grouped GEMM serves in bf16 on the GPU (fused SwiGLU epilogue)
+    "wide": lambda: config([layer(mixer(H=4, G=2, d=32, dv=32, window=40), experts(E=4, top=2, groups=(2, 1), ff=128,
+                                                                                   shared=64)),
+                            layer(mixer(H=4, G=2, d=32, dv=32, window=12), dense(96))], width=256, side=0),
 }
 
 
@@ -422,6 +426,36 @@ def test_plan_grouped_gemm_combine(device, dtype, T, E, top, K, N):
     assert float((got.cpu().double() - want).abs().max()) < tol
     got = moe.combine(y2, wgt.to(device), None)
     assert float((got.cpu().double() - (want - sh.double())).abs().max()) < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,E,top,K,N", [(300, 4, 2, 256, 512), (3, 8, 2, 128, 256), (700, 3, 1, 384, 256)])
+def test_grouped_gemm_on_the_256_tile_kernel(T, E, top, K, N):
+    """Shapes the 256 x 256-tile GEMM serves in grouped mode (bf16, N % 256 == 0, K % 128 == 0):
+    gathered rows in, scattered rows out, experts without rows, row tiles that end inside a
+    tile, and the SwiGLU epilogue over interleaved gate / up rows."""
+    torch.manual_seed(T)
+    idx = torch.stack([torch.randperm(E)[:top] for _ in range(T)]).to(torch.int32)
+    if E > 2:
+        idx[idx == 1] = 0 if top == 1 else idx[idx == 1]  # top 1: expert 1 gets no rows
+    order, offsets = moe.plan(idx.cuda(), E)
+    flat, o = idx.reshape(-1).long(), order.cpu().long()
+    a = torch.randn(T, K).bfloat16()
+    w1 = (torch.randn(E, N, K) * K ** -0.5).bfloat16()
+    assert moe.tile_gemm_ok(a.cuda(), w1.cuda())
+    y1 = moe.grouped_gemm(a.cuda(), w1.cuda(), order, offsets, top, gather=True, scatter=False)
+    want1 = torch.stack([a[s // top].double() @ w1[flat[s]].double().t() for s in o.tolist()])
+    assert float((y1.cpu().double() - want1).abs().max()) < 3e-2
+    g, u = want1[:, :N // 2], want1[:, N // 2:]
+    y1g = moe.grouped_gemm(a.cuda(), moe.interleave_glu(w1.cuda()), order, offsets, top, gather=True, scatter=False,
+                           glu=True)
+    assert float((y1g.cpu().double() - g * torch.sigmoid(g) * u).abs().max()) < 3e-2
+    w2 = (torch.randn(E, N, K) * K ** -0.5).bfloat16()
+    b = torch.randn(T * top, K).bfloat16()  # rows already in sorted order
+    y2 = moe.grouped_gemm(b.cuda(), w2.cuda(), order, offsets, top, gather=False, scatter=True)
+    want2 = torch.empty(T * top, N, dtype=F64)
+    want2[o] = torch.stack([b[r].double() @ w2[flat[s]].double().t() for r, s in enumerate(o.tolist())])
+    assert float((y2.cpu().double() - want2).abs().max()) < 3e-2
 
 
 # ----------------------------------------------------------------- the model in the engine
