@@ -37,6 +37,7 @@ import torch
 from ..ops import mixers as mx
 from ..ops import moe
 from .config import LayeredConfig
+from .gemm_tuning import planned_mm, tune_small_m
 from .llama import AttnMeta, TPGroup
 
 MLP_KINDS = ("dense", "moe")
@@ -80,6 +81,7 @@ class BolinexForCausalLM:
         self.kv_amax = None
         self.layer_hook = None
         self.gemm_plan: dict = {}
+        self.gemm_tuned: set = set()
         # debugging: when a list, forward() appends the residual after every layer
         self.trace_layers: list | None = None
 
@@ -90,8 +92,19 @@ class BolinexForCausalLM:
     def fold_norms(self) -> bool:
         return False
 
+    #: dense projections of a layer, by the name of their weight
+    LINEARS = ("w_in", "w_o", "w_up", "w_down", "w_sgu", "w_sdown", "side_gate", "side_proj")
+
     def tune_gemms(self, sizes, **kw) -> list:
-        return []
+        """Decode batch sizes: the hand-written small-M GEMMs where they beat the
+        library (bf16 on the GPU; models/gemm_tuning.py)."""
+        if self.device.type != "cuda" or self.dtype != torch.bfloat16 or not self.layers:
+            return []
+        groups = [[L[n] for L in self.layers if L.get(n) is not None] for n in self.LINEARS]
+        return tune_small_m([g for g in groups if g], sizes, self.gemm_plan, self.gemm_tuned, **kw)
+
+    def _mm(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        return planned_mm(self.gemm_plan, x, w)
 
     def tune_prefill_gemms(self, max_tokens, **kw) -> list:
         return []
@@ -105,7 +118,7 @@ class BolinexForCausalLM:
         GEMM library loads its kernels for the size before serving)."""
         seen = set()
         for L in self.layers:
-            for name in ("w_in", "w_o", "w_up", "w_down", "w_sgu", "w_sdown", "side_gate", "side_proj"):
+            for name in self.LINEARS:
                 w = L.get(name)
                 if w is None or tuple(w.shape) in seen:
                     continue
@@ -273,7 +286,7 @@ class BolinexForCausalLM:
     def _mix(self, L: dict, h: torch.Tensor, meta: AttnMeta, kc, vc, seq, tables, bs: int, firsts: dict, i: int):
         m, T = L["m"], h.shape[0]
         H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-        p = torch.matmul(h, L["w_in"].t())
+        p = self._mm(h, L["w_in"])
         k_off, v_off, g_off = H * d, (H + G) * d, (H + G) * d + G * dv
         v_own = p[:, v_off:v_off + G * dv]
         firsts[i] = v_own  # the values as projected, for the layers that mix them in
@@ -286,14 +299,14 @@ class BolinexForCausalLM:
                          "window" if size else "causal", size, self._parts(T, H, H // G, size, meta), False, *tl,
                          softcap=float(m.get("softcap") or 0.0), dist_bias=L["bias"])
         a = mx.act_mul(p[:, g_off:g_off + H * dv], a.view(T, H * dv), "sigmoid")
-        return torch.matmul(a, L["w_o"].t())
+        return self._mm(a, L["w_o"])
 
     def _ff(self, L: dict, h: torch.Tensor) -> torch.Tensor | None:
         mlp = L["mlp"]
         if not mlp:
             return None
         if mlp["kind"] == "dense":
-            return torch.matmul(mx.act_mul(torch.matmul(h, L["w_up"].t()), None, "relu2"), L["w_down"].t())
+            return self._mm(mx.act_mul(self._mm(h, L["w_up"]), None, "relu2"), L["w_down"])
         r = mlp["router"]
         gr = r.get("groups") or {"count": 1, "keep": 1}
         z = torch.matmul(h.float(), L["router"].t())
@@ -307,7 +320,7 @@ class BolinexForCausalLM:
         y = moe.grouped_gemm(act, L["w_edown"], order, offsets, r["top"], gather=False, scatter=True)
         shared = None
         if "w_sgu" in L:
-            shared = torch.matmul(mx.glu_act(torch.matmul(h, L["w_sgu"].t()), "silu"), L["w_sdown"].t())
+            shared = self._mm(mx.glu_act(self._mm(h, L["w_sgu"]), "silu"), L["w_sdown"])
         return moe.combine(y, w, shared)
 
     def forward(self, input_ids: torch.Tensor, meta: AttnMeta, kv_caches: list[tuple]) -> torch.Tensor:
@@ -341,8 +354,8 @@ class BolinexForCausalLM:
                 _, xa = mx.residual_step(X, ym, yf, eps=eps, out_dtype=dt, want_cast=dt != torch.float32)
                 xa = X if xa is None else xa
                 sd_ = self.side_dim
-                g = mx.act_mul(torch.matmul(xa, L["side_gate"].t()), side[:, i * sd_:(i + 1) * sd_], "gelu_tanh")
-                y = torch.matmul(g, L["side_proj"].t())
+                g = mx.act_mul(self._mm(xa, L["side_gate"]), side[:, i * sd_:(i + 1) * sd_], "gelu_tanh")
+                y = self._mm(g, L["side_proj"])
                 if last and self.trace_layers is None:
                     ysel = y  # joins the residual with the final norm, on the chosen rows only
                 else:
