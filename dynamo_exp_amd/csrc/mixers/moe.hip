@@ -108,19 +108,26 @@ __global__ void __launch_bounds__(64 * kRouteWaves) moe_route_kernel(int* __rest
 // order [R]: slots sorted by expert, stable; offsets [E + 1].  One workgroup:
 // counts by LDS atomics (the counts do not depend on their order), a serial
 // scan over the experts, then every wave places the slots of its experts in
-// slot order with ballots.
+// slot order with ballots.  STAGE: the choices are first copied into LDS as
+// bytes (E <= 256, R <= kPlanStage), so the placement passes read no global
+// memory.
 constexpr int kPlanThreads = 1024;
+constexpr int kPlanStage = 48 * 1024;
+template <bool STAGE>
 __global__ void __launch_bounds__(kPlanThreads) moe_plan_kernel(int* __restrict__ order, int* __restrict__ offsets,
                                                                 const int* __restrict__ idx, int R, int E) {
   extern __shared__ int ism[];
   int* cnt = ism;
   int* base = ism + E;
+  unsigned char* mine = reinterpret_cast<unsigned char*>(ism + 2 * E + 1);
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   for (int e = tid; e < E; e += kPlanThreads) cnt[e] = 0;
   __syncthreads();
   for (int r = tid; r < R; r += kPlanThreads) {
     const int e = idx[r];
-    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    const bool ok = e >= 0 && e < E;
+    if (ok) atomicAdd(&cnt[e], 1);
+    if constexpr (STAGE) mine[r] = ok ? (unsigned char)e : 0;  // choices outside the experts are rejected by route
   }
   __syncthreads();
   if (tid == 0) {
@@ -137,7 +144,9 @@ __global__ void __launch_bounds__(kPlanThreads) moe_plan_kernel(int* __restrict_
     int at = base[e];
     for (int r0 = 0; r0 < R; r0 += 64) {
       const int r = r0 + lane;
-      const bool hit = r < R && idx[r] == e;
+      bool hit;
+      if constexpr (STAGE) hit = r < R && mine[r] == e;
+      else hit = r < R && idx[r] == e;
       const unsigned long long m = __builtin_amdgcn_ballot_w64(hit);
       if (hit) order[at + __builtin_popcountll(m & ((1ull << lane) - 1ull))] = r;
       at += __builtin_popcountll(m);
@@ -291,25 +300,52 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(T* __restrict__ out, 
   }
 }
 
-// out[t, :] = sum_k wgt[t, k] * y[t * top + k, :] (+ shared[t, :]), fp32 sum in the order of k
-template <typename T>
+// out[t, :] = sum_k wgt[t, k] * y[t * top + k, :] (+ shared[t, :]), fp32 sum in the order of k;
+// V elements (16 bytes) per thread and access, V = 1 for unaligned widths
+template <typename T, int V>
 __global__ void __launch_bounds__(256) moe_combine_kernel(T* __restrict__ out, const T* __restrict__ y,
                                                           const float* __restrict__ wgt, const T* __restrict__ shared,
                                                           int64_t sh_stride, int top, int W) {
   const int64_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < W; c += 256) {
-    float acc = 0.f;
+  auto load = [](const T* p, float* f) {
+    if constexpr (V == 1) {
+      if constexpr (sizeof(T) == 2) f[0] = bf16_to_f32(p[0]); else f[0] = p[0];
+    } else if constexpr (sizeof(T) == 2) {
+      const u16x8 a = *reinterpret_cast<const u16x8*>(p);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[2 * i] = bf16lo(a.w[i]), f[2 * i + 1] = bf16hi(a.w[i]);
+    } else {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = a[i];
+    }
+  };
+  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+    float acc[V], f[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
     for (int k = 0; k < top; ++k) {
-      const T v = y[(t * top + k) * (int64_t)W + c];
-      float f;
-      if constexpr (sizeof(T) == 2) f = bf16_to_f32(v); else f = v;
-      acc += wgt[t * top + k] * f;
+      load(y + (t * top + k) * (int64_t)W + c, f);
+      const float g = wgt[t * top + k];
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += g * f[i];
     }
     if (shared) {
-      const T v = shared[t * sh_stride + c];
-      if constexpr (sizeof(T) == 2) acc += bf16_to_f32(v); else acc += v;
+      load(shared + t * sh_stride + c, f);
+#pragma unroll
+      for (int i = 0; i < V; ++i) acc[i] += f[i];
     }
-    if constexpr (sizeof(T) == 2) out[t * (int64_t)W + c] = f32_to_bf16(acc); else out[t * (int64_t)W + c] = acc;
+    T* o = out + t * (int64_t)W + c;
+    if constexpr (V == 1) {
+      if constexpr (sizeof(T) == 2) o[0] = f32_to_bf16(acc[0]); else o[0] = acc[0];
+    } else if constexpr (sizeof(T) == 2) {
+      u16x8 r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r.w[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
+      *reinterpret_cast<u16x8*>(o) = r;
+    } else {
+      *reinterpret_cast<f32x4*>(o) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    }
   }
 }
 
@@ -334,8 +370,11 @@ int dxm_moe_route(int* idx, float* w, const float* z, const float* corr, int T, 
 int dxm_moe_plan(int* order, int* offsets, const int* idx, int R, int E, hipStream_t st) {
   if (E < 1 || R < 0) return 1;
   const size_t lds = (size_t)(2 * E + 1) * sizeof(int);
-  if (lds > 48 * 1024) return 2;
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kPlanThreads), lds, st, order, offsets, idx, R, E);
+  if (lds > 12 * 1024) return 2;
+  if (E <= 256 && R <= kPlanStage)
+    hipLaunchKernelGGL(moe_plan_kernel<true>, dim3(1), dim3(kPlanThreads), lds + R, st, order, offsets, idx, R, E);
+  else
+    hipLaunchKernelGGL(moe_plan_kernel<false>, dim3(1), dim3(kPlanThreads), lds, st, order, offsets, idx, R, E);
   DX_CHECK_LAUNCH();
   return 0;
 }
@@ -361,12 +400,24 @@ int dxm_moe_combine(void* out, const void* y, const float* wgt, const void* shar
                     int W, int f32, hipStream_t st) {
   if (T <= 0) return 0;
   if (top < 1 || W < 1) return 1;
-  if (f32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(T), dim3(256), 0, st, (float*)out, (const float*)y, wgt,
-                       (const float*)shared, sh_stride, top, W);
-  else
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)y, wgt,
-                       (const bf16_t*)shared, sh_stride, top, W);
+  const int per = f32 ? 4 : 8;  // elements per 16 bytes
+  const bool vec = W % per == 0 && sh_stride % per == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)y % 16 == 0 &&
+                   (uintptr_t)shared % 16 == 0;
+  if (f32) {
+    if (vec)
+      hipLaunchKernelGGL((moe_combine_kernel<float, 4>), dim3(T), dim3(256), 0, st, (float*)out, (const float*)y, wgt,
+                         (const float*)shared, sh_stride, top, W);
+    else
+      hipLaunchKernelGGL((moe_combine_kernel<float, 1>), dim3(T), dim3(256), 0, st, (float*)out, (const float*)y, wgt,
+                         (const float*)shared, sh_stride, top, W);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((moe_combine_kernel<bf16_t, 8>), dim3(T), dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)y,
+                         wgt, (const bf16_t*)shared, sh_stride, top, W);
+    else
+      hipLaunchKernelGGL((moe_combine_kernel<bf16_t, 1>), dim3(T), dim3(256), 0, st, (bf16_t*)out, (const bf16_t*)y,
+                         wgt, (const bf16_t*)shared, sh_stride, top, W);
+  }
   DX_CHECK_LAUNCH();
   return 0;
 }

@@ -237,10 +237,11 @@ class BolinexForCausalLM:
             out = dict(m=m, norm_w=f32(sd[f"l{i}.norm1"]), norm_b=f32(sd[f"l{i}.norm1.b"]),
                        w_in=act(p + "q", p + "k", p + "v", p + "g"), w_o=act(p + "o"),
                        bias=(f32(sd[p + "r1"]), f32(sd[p + "r2"])) if p + "r1" in sd else None,
-                       mix_from=None, lam=0.0)
+                       mix_from=None, mix_source=False, lam=0.0)
             if m.get("v_mix"):
                 if first_vmix is None:
                     first_vmix = i
+                    out["mix_source"] = True
                 else:
                     out.update(mix_from=first_vmix, lam=float(sd[p + "vmix"].float()))
             mlp, q = L.get("mlp"), f"l{i}.mlp."
@@ -288,8 +289,8 @@ class BolinexForCausalLM:
         H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         p = self._mm(h, L["w_in"])
         k_off, v_off, g_off = H * d, (H + G) * d, (H + G) * d + G * dv
-        v_own = p[:, v_off:v_off + G * dv]
-        firsts[i] = v_own  # the values as projected, for the layers that mix them in
+        if L["mix_source"]:  # the values as projected stay alive for the layers that mix them in
+            firsts[i] = p[:, v_off:v_off + G * dv]
         vf = firsts[L["mix_from"]] if L["mix_from"] is not None else None
         mx.headprep_cache(p, meta.positions, meta.slot_mapping, 0, G, d, k_off, None, None, self.cfg.rms_norm_eps,
                           None, kc, vc, v_mode=2, v_off=v_off, v_w=G * dv, v_first=vf, v_lambda=L["lam"])

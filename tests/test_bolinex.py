@@ -392,6 +392,20 @@ def test_route_alone(device, E, top, groups):
     assert torch.equal(gi.cpu().long(), idx)
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("T,E,top", [(26000, 5, 2), (50, 300, 3), (8192, 8, 2), (1, 1, 1)])
+def test_plan_sizes(device, T, E, top):
+    """More slots than the kernel stages in LDS, more experts than a byte counts, a usual prompt step."""
+    g = torch.Generator().manual_seed(T)
+    idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(min(T, 64))]).to(torch.int32)
+    idx = idx.repeat(-(-T // idx.shape[0]), 1)[:T].contiguous()
+    idx[::7] = idx[::7].flip(1)
+    order, offsets = moe.plan(idx.to(device), E)
+    flat = idx.reshape(-1).long()
+    assert torch.equal(order.cpu().long(), torch.sort(flat, stable=True).indices)
+    assert offsets.cpu().tolist() == [0] + torch.bincount(flat, minlength=E).cumsum(0).tolist()
+
+
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("T,E,top,K,N", [(1, 3, 1, 16, 8), (37, 5, 2, 70, 33), (150, 4, 3, 96, 130), (70, 16, 1, 64, 64)])
 def test_plan_grouped_gemm_combine(device, dtype, T, E, top, K, N):
