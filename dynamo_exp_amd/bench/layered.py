@@ -145,7 +145,7 @@ def attention_kernels(s: dict, L: int, B: int) -> dict:
     vc = torch.randn_like(kc)
     q = torch.randn(B, H * d, device=dev, dtype=dt)
     pos = torch.full((B,), L - 1, device=dev)
-    parts = mx.row_attention_parts(B, G, L)
+    parts = mx.row_attention_parts(B, G, L, mx.GROUP_TARGET_WAVES)
     us = _timed(lambda: mx.attention(q, kc, vc, pos, None, bt, bs, H, 1, H // G, d, d, d ** -0.5, "causal", 0, parts))
     res["bekulix_decode"] = {"us": round(us, 1), "TB/s": round(byts / us / 1e6, 2), "parts": parts}
     kl = torch.randn(nbb, G, bs, d, device=dev, dtype=dt)
@@ -236,7 +236,7 @@ def bolinex_kernels(s: dict, L: int, B: int, T: int) -> dict:
     vcd = torch.randn_like(kcd)
     qd = torch.randn(B, H * d, device=dev, dtype=dt)
     posd = torch.full((B,), L - 1, device=dev)
-    parts = mx.row_attention_parts(B, G, win)
+    parts = mx.row_attention_parts(B, G, win, mx.GROUP_TARGET_WAVES)
     for name, kw in (("plain", {}), ("cap_penalty", dict(softcap=30.0, dist_bias=(r1, r2)))):
         us = _timed(lambda: mx.attention(qd, kcd, vcd, posd, None, btd, bs, H, 1, H // G, d, d, d ** -0.5, "window", win,
                                          parts, **kw))

@@ -282,7 +282,9 @@ class BolinexForCausalLM:
         if meta.is_prefill:
             rows -= meta.num_prefill_tokens if self.dtype == torch.bfloat16 and self.device.type == "cuda" else 0
         units = H if self.dtype != torch.bfloat16 else max(1, H // group) * (-(-group // 32))
-        return mx.row_attention_parts(max(rows, 1), units, vis)
+        grouped = self.dtype == torch.bfloat16 and self.device.type == "cuda"
+        return mx.row_attention_parts(max(rows, 1), units, vis,
+                                      mx.GROUP_TARGET_WAVES if grouped else mx.ROW_TARGET_WAVES)
 
     def _mix(self, L: dict, h: torch.Tensor, meta: AttnMeta, kc, vc, seq, tables, bs: int, firsts: dict, i: int):
         m, T = L["m"], h.shape[0]

@@ -31,6 +31,9 @@ MAX_STREAMS = 8
 # into parts shorter than ROW_MIN_PART
 ROW_TARGET_WAVES = 2048
 ROW_MIN_PART = 128
+# grouped decode kernel: one wave per workgroup, four workgroups resident per CU (LDS), so
+# about 1024 waves fill the chip once; more parts only add merge work
+GROUP_TARGET_WAVES = 1024
 
 
 def _m():
@@ -283,13 +286,13 @@ def headprep_cache(x: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor
 
 
 # ----------------------------------------------------------------- attention
-def row_attention_parts(rows: int, n_qh: int, max_visible: int) -> int:
-    """Key partitions per row so a launch has about ROW_TARGET_WAVES waves
-    (n_qh: the independent units per row -- query heads for the row kernel, K
-    heads for the grouped decode kernel)."""
+def row_attention_parts(rows: int, n_qh: int, max_visible: int, target: int = ROW_TARGET_WAVES) -> int:
+    """Key partitions per row so a launch has about `target` waves (n_qh: the
+    independent units per row -- query heads for the row kernel, K heads for
+    the grouped decode kernel, whose target is GROUP_TARGET_WAVES)."""
     if rows <= 0:
         return 1
-    want = -(-ROW_TARGET_WAVES // (rows * n_qh))
+    want = -(-target // (rows * n_qh))
     return max(1, min(want, max_visible // ROW_MIN_PART))
 
 
